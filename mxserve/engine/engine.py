@@ -46,7 +46,9 @@ class LLMEngine:
         self.args = args
         self.model_config = get_model_config(args.model)
         self.runner = ModelRunner(args, self.model_config)
-        self.kv = KVCacheManager(self.runner.num_blocks, args.block_size, args.enable_prefix_caching)
+        # a cached prefix block carries no recurrent state to resume from: such models recompute
+        self.kv = KVCacheManager(self.runner.num_blocks, args.block_size,
+                                 args.enable_prefix_caching and not self.model_config.has_recurrent_state)
         self.scheduler = Scheduler(self.kv, args.max_num_seqs, args.max_num_batched_tokens, args.max_model_len,
                                    args.enable_chunked_prefill)
         self.requests: dict[str, Request] = {}

@@ -49,7 +49,7 @@ class InputBuffers:
     device views (stable addresses)."""
 
     _SEGS = (("input_ids", np.int64, "T"), ("positions", np.int64, "T"), ("slot_mapping", np.int64, "T"),
-             ("logits_indices", np.int64, "S"), ("seeds", np.int64, "S"), ("steps", np.int64, "S"),
+             ("logits_indices", np.int64, "T"), ("seeds", np.int64, "S"), ("steps", np.int64, "S"),
              ("srows", np.int64, "S"), ("trow", np.int64, "T"),
              ("bt_idx", np.int64, "U"), ("seq_lens", np.int32, "S"), ("qsl", np.int32, "S1"),
              ("rows", np.int32, "S"), ("sseq", np.int32, "S"), ("top_k", np.int32, "S"), ("bt_val", np.int32, "U"),
@@ -109,7 +109,7 @@ class ModelRunner:
         self.dtype = _DTYPES[args.dtype] if self.is_gpu else torch.float32
         self.bs = args.block_size
         t0 = time.time()
-        self.model = build_model(cfg, self.device, self.dtype, args.moe_dispatch)
+        self.model = build_model(cfg, self.device, self.dtype, args.moe_dispatch, self.bs)
         self.weight_source = load_weights(self.model, args.load_format, args.seed)
         log.info("weights (%s) ready in %.1fs", self.weight_source, time.time() - t0)
         self.max_blocks_per_seq = math.ceil(args.max_model_len / self.bs)
@@ -128,13 +128,18 @@ class ModelRunner:
                                          max_rows=args.max_num_batched_tokens + args.max_num_seqs)
         self.num_blocks = self._determine_num_blocks()
         m = self.model
-        self.kv_cache = torch.zeros(self.num_blocks, cfg.num_layers, 2, m.nkv, self.bs, cfg.head_dim,
-                                    dtype=self.kv_dtype, device=self.device)
+        self.kv_cache = torch.zeros(m.kv_cache_shape(self.num_blocks, self.bs), dtype=self.kv_dtype,
+                                    device=self.device)
         self.block_bytes = self.kv_cache[0].numel() * self.kv_cache.element_size()
         # block tables live on the device, one persistent row per live request, updated
         # incrementally (a decode step touches at most one new entry per request)
         n_rows = args.max_num_seqs + 8
         self.bt_dev = torch.zeros(n_rows, self.max_blocks_per_seq, dtype=torch.int32, device=self.device)
+        # recurrent layers (linear attention, mLSTM): one fp32 state slot per row, every layer's state
+        # in it.  A slot is not cleared when its row goes to another request: a sequence's first
+        # tokens (position 0) start from zero inside the kernels, whatever the slot holds.
+        self.state = (torch.zeros(n_rows, m.state_floats, dtype=torch.float32, device=self.device)
+                      if m.state_floats else None)
         # last sampled token per row: a decode whose input was sampled by a step still in flight
         # (async scheduling) reads it here on the device
         self.last_tok = torch.zeros(n_rows, dtype=torch.int64, device=self.device)
@@ -201,7 +206,7 @@ class ModelRunner:
 
     def _local_num_blocks(self) -> int:
         a, c, m = self.args, self.cfg, self.model
-        per_block = c.num_layers * 2 * m.nkv * self.bs * c.head_dim * torch.empty(0, dtype=self.kv_dtype).element_size()
+        per_block = math.prod(m.kv_cache_shape(1, self.bs)) * torch.empty(0, dtype=self.kv_dtype).element_size()
         if a.num_gpu_blocks:
             return int(a.num_gpu_blocks)
         if not self.is_gpu:
@@ -211,6 +216,7 @@ class ModelRunner:
         # activation workspace for the largest step + logits + graph pools
         act = a.max_num_batched_tokens * (c.hidden_size * 12 + 2 * c.intermediate_size // m.tp_size) * 2
         act += a.max_num_seqs * c.vocab_size * 4 * 3 + (2 << 30)
+        act += (a.max_num_seqs + 8) * m.state_floats * 4  # recurrent state slots
         budget = int(total * a.gpu_memory_utilization) - (total - free) - act
         n = max(64, budget // per_block)
         log.info("KV pool: %d blocks x %.1f KiB = %.1f GB (%d tokens)", n, per_block / 1024, n * per_block / 1e9,
@@ -306,13 +312,23 @@ class ModelRunner:
             if s.sample:
                 sample_rows.append(nd + i)
                 steps.append(s.out_idx)
+        # scoring steps (SchedulerOutput.score): logits of chosen rows of each chunk and no sampling.  A
+        # decode-only step that replays a graph keeps the graph's own rows (one per sequence).
+        n_score = None
+        if getattr(so, "score", False) and not graph_bs:
+            idx = [qsl[j] + o for j, s in enumerate(so.all()) for o in (s.logit_offsets or ())]
+            n_score = len(idx)
+            sample_rows, steps = [], []
         rows_np = np.asarray(rows, dtype=np.int32)
         h["seq_lens"][:S] = lens
         h["qsl"][:S + 1] = qsl
         h["rows"][:S] = rows_np
         ns = len(sample_rows)
         srows = rows_np[sample_rows] if ns != S else rows_np
-        h["logits_indices"][:ns] = np.asarray(qsl, dtype=np.int64)[np.asarray(sample_rows, dtype=np.int64) + 1] - 1
+        if n_score is not None:
+            h["logits_indices"][:n_score] = idx
+        else:
+            h["logits_indices"][:ns] = np.asarray(qsl, dtype=np.int64)[np.asarray(sample_rows, dtype=np.int64) + 1] - 1
         h["temperature"][:ns] = self._row_temp[srows]
         h["top_p"][:ns] = self._row_topp[srows]
         h["top_k"][:ns] = self._row_topk[srows]
@@ -353,7 +369,8 @@ class ModelRunner:
                 lp = (sel.tolist(), int(lpk[sel].max()))
         hist_init, self._hist_init = self._hist_init, []
         return dict(S=S, T=T, nd=nd, max_q=max_q, max_seq=max(lens), sample_rows=sample_rows, U=U,
-                    big_update=big_update, graph_bs=graph_bs, lp=lp, pen=use_pen, hist_init=hist_init)
+                    big_update=big_update, graph_bs=graph_bs, lp=lp, pen=use_pen, hist_init=hist_init,
+                    n_score=n_score)
 
     def _upload(self, meta: dict) -> None:
         self.buf.upload()
@@ -397,6 +414,15 @@ class ModelRunner:
             _fault_injection(self._steps, tp.tp_rank)
         ids = self.execute_host(meta)
         handle = {"so": so, "rows": meta["sample_rows"]}
+        if getattr(so, "score", False):
+            # the asked rows' logits stay on the device; the caller reads them (engine/replay.py)
+            lg = self._logits
+            if gbs:  # a replayed graph computed one row per sequence: keep those that were asked for
+                want = [j for j, s in enumerate(so.all()) if s.logit_offsets]
+                lg = lg.index_select(0, torch.tensor(want, dtype=torch.int64).to(self.device)) if want else None
+            handle["logits"] = lg
+            handle["rows"] = []
+            return handle
         if car is not None:
             # every TP step, sampling or not: a fault is caught at the step that contains it
             self._err_slot ^= 1
@@ -555,7 +581,11 @@ class ModelRunner:
 
     def _forward_eager(self, meta: dict, sample: bool):
         S, T, nd = meta["S"], meta["T"], meta["nd"]
+        n_score = meta.get("n_score")
         v = self._views(S, T, len(meta["sample_rows"]))
+        if n_score is not None:
+            v["logits_indices"] = self.buf.d["logits_indices"][:n_score]
+            v["sseq"] = None  # every layer computes every row
         bt = self.bt_dev.index_select(0, v["rows"].long())
         pq = None
         if S > nd:
@@ -564,13 +594,16 @@ class ModelRunner:
                           seq_lens=v["seq_lens"], query_start_loc=v["qsl"], logits_indices=v["logits_indices"],
                           num_decodes=nd, num_prefills=S - nd, num_prefill_tokens=T - nd,
                           max_query_len=meta["max_q"], max_seq_len=meta["max_seq"], prefill_query_start_loc=pq,
-                          sample_seq=v["sseq"])
+                          sample_seq=v["sseq"], state_rows=v["rows"], state=self.state)
         inp = v["input_ids"]
         if nd:
             d_in = inp[:nd]
             d_in.copy_(torch.where(d_in < 0, self.last_tok.index_select(0, v["rows"][:nd].long()), d_in))
         self._write_hist(v, inp)
         hidden = self.model.forward(inp, md, self.kv_cache)
+        if n_score is not None:
+            self._logits = self.model.compute_logits(hidden) if n_score else None
+            return None
         if not sample:
             return None
         logits = self.model.compute_logits(hidden)
@@ -593,7 +626,7 @@ class ModelRunner:
             positions=v["positions"], slot_mapping=v["slot_mapping"], block_tables=bt,
             seq_lens=v["seq_lens"], query_start_loc=v["qsl"], logits_indices=self._arange[:b],
             num_decodes=b, num_prefills=0, num_prefill_tokens=0, max_query_len=1,
-            max_seq_len=self.args.max_model_len)
+            max_seq_len=self.args.max_model_len, state_rows=v["rows"], state=self.state)
         hidden = self.model.forward(inp, md, self.kv_cache)
         logits = self.model.compute_logits(hidden)
         self._penalize(v, logits)  # rows with neutral penalties exit at once
@@ -611,7 +644,7 @@ class ModelRunner:
         if not buckets:
             log.warning("no decode bucket has graph-capturable collectives; decode runs eagerly")
             return
-        if tune:
+        if tune and "l0.qkv" in m.w:  # the transformer families' projections
             self._tune_gemms(buckets)
         self._capture(buckets)
 
@@ -724,7 +757,7 @@ class ModelRunner:
             torch.cuda.synchronize(self.device)
         self.graphs.clear()
         self._logits = None
-        for name in ("kv_cache", "model", "bt_dev", "last_tok", "hist", "_pen_counts", "buf"):
+        for name in ("kv_cache", "state", "model", "bt_dev", "last_tok", "hist", "_pen_counts", "buf"):
             setattr(self, name, None)
 
     def kv_stats(self) -> dict:

@@ -26,6 +26,8 @@ class ScheduledReq:
     sample: bool
     start: int = 0  # first position computed by this chunk
     out_idx: int = 0  # index of the output token this chunk samples (RNG counter)
+    # scoring steps: offsets inside this chunk whose logits the caller wants (no token is sampled)
+    logit_offsets: Optional[list] = None
 
 
 @dataclass
@@ -33,6 +35,7 @@ class SchedulerOutput:
     decodes: list = field(default_factory=list)  # ScheduledReq, 1 token each
     prefills: list = field(default_factory=list)  # ScheduledReq, chunk of >=1 token
     preempted: list = field(default_factory=list)
+    score: bool = False  # a scoring step: logits of chosen rows, nothing sampled (schedule_forced)
 
     @property
     def num_tokens(self) -> int:
@@ -237,6 +240,38 @@ class Scheduler:
                 s.out_idx = len(r.output_token_ids) + r.num_pending
                 r.num_pending += 1
         return out
+
+    # ------------------------------------------------------------------ forced steps (replay, scoring)
+    def admit_forced(self, req: Request) -> None:
+        """A request whose tokens the caller feeds step by step joins the running set at once."""
+        if self.num_slots_used() >= self.max_num_seqs:
+            raise RuntimeError(f"{self.max_num_seqs} requests are live already")
+        req.status = Status.RUNNING
+        req.scheduled_time = time.monotonic()
+        self.running.append(req)
+        self.num_added += 1
+
+    def schedule_forced(self, plan: list) -> SchedulerOutput:
+        """A step the caller dictates: plan = [(request, new tokens, logit offsets)], the new tokens
+        already appended to the request's known tokens.  Same block allocation and the same batch
+        order as schedule() (single tokens of started sequences first, chunks after); no policy, no
+        preemption: a pool too small for the plan is an error.  Nothing is sampled."""
+        out = SchedulerOutput(score=True)
+        for req, n, offsets in plan:
+            if n <= 0 or req.num_computed_tokens + n > req.num_known_tokens:
+                raise ValueError(f"{req.request_id}: {n} new tokens do not fit its {req.num_known_tokens} known ones")
+            if not self.kv.allocate_slots(req, n):
+                raise RuntimeError(f"KV pool exhausted: {req.request_id} needs blocks for {n} more tokens "
+                                   f"({self.kv.num_free()} blocks free)")
+            s = ScheduledReq(req, n, False, start=req.num_computed_tokens, logit_offsets=list(offsets or ()))
+            (out.decodes if n == 1 and s.start > 0 else out.prefills).append(s)
+            req.num_computed_tokens += n
+        return out
+
+    def finish_forced(self, req: Request) -> None:
+        if req in self.running:
+            self.running.remove(req)
+        self._finish(req, Status.FINISHED_STOPPED)
 
     # ------------------------------------------------------------------ update
     def update(self, out: SchedulerOutput, sampled: dict[str, int]) -> list[Request]:

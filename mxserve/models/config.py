@@ -18,7 +18,7 @@ from typing import Optional
 @dataclass
 class ModelConfig:
     name: str
-    arch: str  # "llama" | "qwen3" | "mixtral"
+    arch: str  # "llama" | "qwen3" | "mixtral" | "voletar"
     hidden_size: int
     intermediate_size: int
     num_layers: int
@@ -40,10 +40,20 @@ class ModelConfig:
     bos_token_id: Optional[int] = None
     eos_token_ids: list = field(default_factory=list)
     chat_template: str = "llama3"
+    # designs whose layers differ from one another (arch "voletar"): the checkpoint's own config.json
+    # structure -- per-layer mixer type and sizes, the looped span, norm eps, logit soft-cap -- as
+    # mxserve/models/voletar.py reads it.  None for the uniform transformer families.
+    arch_config: Optional[dict] = None
 
     @property
     def is_moe(self) -> bool:
         return self.num_experts > 0
+
+    @property
+    def has_recurrent_state(self) -> bool:
+        """Layers that carry a per-sequence state from token to token (linear attention, mLSTM): no
+        prefix caching (a cached block has no state to resume from) and one state slot per request."""
+        return self.arch == "voletar"
 
     @property
     def q_size(self) -> int:
@@ -54,9 +64,15 @@ class ModelConfig:
         return self.num_kv_heads * self.head_dim
 
     def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
+        if self.arch_config is not None:
+            from .voletar import layer_plan
+            return sum(r.kv_heads * (r.dk + r.dv) for r in layer_plan(self.arch_config).attn_runs) * dtype_bytes
         return self.num_layers * 2 * self.num_kv_heads * self.head_dim * dtype_bytes
 
     def num_params(self) -> int:
+        if self.arch_config is not None:
+            from .voletar import weight_shapes
+            return sum(int(__import__("math").prod(v)) for v in weight_shapes(self.arch_config).values())
         h, i, L = self.hidden_size, self.intermediate_size, self.num_layers
         attn = h * (self.q_size + 2 * self.kv_size) + self.q_size * h
         if self.is_moe:
@@ -150,7 +166,27 @@ _reg(ModelConfig(
     max_position_embeddings=8192, bos_token_id=1, eos_token_ids=[2], chat_template="llama3"))
 
 
+def voletar_config(name: str, d: dict) -> ModelConfig:
+    """A Voletar checkpoint's config.json: `width`, `vocab`, `layers` (each with `type`, `mixer`, `mlp`),
+    optional `loop` {start, stop, times}, `norm.eps`, optional `logit_softcap`.  The uniform fields are
+    filled from the first layer for the code that sizes things from them (profiler, planner)."""
+    layers = d["layers"]
+    mx = layers[0]["mixer"]
+    att = mx.get("left", mx)
+    ffs = [l["mlp"]["ff"] for l in layers if l.get("mlp")]
+    keep = {k: d[k] for k in ("layers", "loop", "norm", "logit_softcap", "width", "vocab") if k in d}
+    return ModelConfig(
+        name=name, arch="voletar", hidden_size=int(d["width"]), intermediate_size=max(ffs) if ffs else 0,
+        num_layers=len(layers), num_heads=int(att["heads"]), num_kv_heads=int(att.get("kv_heads", att["heads"])),
+        head_dim=int(att["dim"]), vocab_size=int(d["vocab"]), rms_norm_eps=float(d.get("norm", {}).get("eps", 1e-5)),
+        tie_word_embeddings=False, max_position_embeddings=int(d.get("max_position_embeddings", 1 << 20)),
+        bos_token_id=d.get("bos_token_id"), eos_token_ids=list(d.get("eos_token_ids") or []),
+        chat_template="chatml", arch_config=keep)
+
+
 def _from_hf_json(name: str, d: dict) -> ModelConfig:
+    if d.get("architecture") == "Voletar":
+        return voletar_config(name, d)
     arch_list = d.get("architectures") or []
     mt = d.get("model_type", "")
     if "qwen3" in mt or any("Qwen3" in a for a in arch_list):

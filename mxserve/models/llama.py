@@ -39,6 +39,9 @@ class AttnMetadata:
     max_seq_len: int
     prefill_query_start_loc: Optional[torch.Tensor] = None  # [P+1] int32, rebased at 0
     sample_seq: Optional[torch.Tensor] = None  # [S_sample] int32: sequence of each logits row
+    # models with recurrent layers: each sequence's slot in the fp32 state pool [slots, state_floats]
+    state_rows: Optional[torch.Tensor] = None  # [S] int32
+    state: Optional[torch.Tensor] = None
 
     @property
     def num_tokens(self) -> int:
@@ -103,6 +106,13 @@ class TransformerLM:
             self.e_local = cfg.num_experts // self.tp_size
             self.e_offset = self.tp_rank * self.e_local
         self.vocab_local = (cfg.vocab_size + self.tp_size - 1) // self.tp_size
+
+    is_recurrent = False
+    state_floats = 0
+
+    def kv_cache_shape(self, num_blocks: int, block_size: int) -> tuple:
+        """The paged pool: block-major, a block holds every layer's K and V."""
+        return (num_blocks, self.cfg.num_layers, 2, self.nkv, block_size, self.cfg.head_dim)
 
     # ------------------------------------------------------------------ weights
     def local_shapes(self) -> dict[str, tuple]:
@@ -503,5 +513,10 @@ def _pad_rows(t: torch.Tensor, n: int) -> torch.Tensor:
     return torch.cat([t, pad])
 
 
-def build_model(cfg: ModelConfig, device, dtype=torch.bfloat16, moe_dispatch: str = "allreduce") -> TransformerLM:
+def build_model(cfg: ModelConfig, device, dtype=torch.bfloat16, moe_dispatch: str = "allreduce",
+                block_size: int = 16):
+    """The model class of a config's architecture."""
+    if cfg.arch == "voletar":
+        from .voletar import VoletarLM
+        return VoletarLM(cfg, device, dtype, block_size)
     return TransformerLM(cfg, device, dtype, moe_dispatch)

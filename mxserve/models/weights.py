@@ -181,7 +181,21 @@ def load_sharded_safetensors(model, model_dir: str) -> int:
 
 
 def load_weights(model, load_format: str = "auto", seed: int = 0) -> str:
-    """Populate `model` (TransformerLM).  Returns the source used: 'safetensors' | 'random'."""
+    """Populate `model`.  Returns the source used: 'safetensors' | 'random'."""
+    if model.cfg.arch == "voletar":  # checkpoint names are the model's own (mxserve/models/voletar.py)
+        model_dir = find_local_model_dir(model.cfg.name)
+        files = sorted(glob.glob(os.path.join(model_dir, "*.safetensors"))) if model_dir else []
+        if load_format in ("auto", "safetensors") and files:
+            from safetensors.torch import load_file
+            full = {}
+            for f in files:
+                full.update(load_file(f))
+            model.load_full_state(full)
+            return "safetensors"
+        if load_format == "safetensors":
+            raise FileNotFoundError(f"no safetensors for {model.cfg.name}")
+        model.init_random(seed=seed)
+        return "random"
     if load_format == "random_full":  # unsharded host init, then shard: identical model for any TP size
         model.load_full_state(random_full_state(model.cfg, seed=seed, std=0.05, dtype=torch.float32))
         return "random_full"
