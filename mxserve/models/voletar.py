@@ -225,7 +225,7 @@ class VoletarLM:
         w, W = self.w, self.width
         ctx = StepContext(md=md, cache=kv_cache, state=md.state, block_size=self.block_size, eps=self.eps)
         x0 = F.embedding(input_ids, w["embed"])
-        x = x0.float()
+        x = x0.to(torch.float32, copy=True)  # fp32 models: never an alias of x0
         T = x.shape[0]
         pending = None
         cat = None

@@ -93,7 +93,7 @@ def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """y = x @ w.T.  Decode-sized GEMMs (M <= decode_gemm.MAX_M) run the hand-written MFMA kernel where the
     tuning pass at graph capture measured it faster than hipBLASLt for that batch bucket and
     projection (mxserve/ops/decode_gemm.py); everything else is hipBLASLt."""
-    if _gpu(x) and x.dim() == 2:
+    if _gpu(x) and x.dim() == 2 and x.dtype == torch.bfloat16:  # fp32 models: the library's fp32 GEMM
         M = x.shape[0]
         from . import decode_gemm
         if M <= decode_gemm.MAX_M:

@@ -3,8 +3,11 @@
 
   mxserve/_rt.so  host runtime (block pool, hashing, KV indexer)          g++ + pybind11
   mxserve/_C.so   gfx950 HIP kernels + KV-transfer agent, torch bindings   hipcc --offload-arch=gfx950
+  mxserve/_M.so   gfx950 mixer kernels (windowed attention, recurrences)   hipcc --offload-arch=gfx950
 
-Incremental (mtime-based) and parallel.  `python setup_ext.py [--clean] [-j N] [--only rt|C]`.
+Incremental (mtime-based) and parallel.  `python setup_ext.py [--clean] [-j N] [--only rt|C|M]`.
+A model loads only the extensions it uses, and builds a missing one on first use: the mixer models
+need _rt and _M, not the larger _C.
 HIP sources are written for CDNA4 directly: hipcc compiles them as-is, nothing is hipified.
 """
 from __future__ import annotations
@@ -36,12 +39,12 @@ def _pybind_includes() -> list[str]:
     return [f"-I{pybind11.get_include()}", f"-I{sysconfig.get_paths()['include']}"]
 
 
-def _torch_flags():
+def _torch_flags(name: str = "_C"):
     import torch
     from torch.utils import cpp_extension as ce
     inc = [f"-I{p}" for p in ce.include_paths(device_type="cuda")]
     abi = int(torch._C._GLIBCXX_USE_CXX11_ABI)
-    defs = ["-DTORCH_API_INCLUDE_EXTENSION_H", "-DTORCH_EXTENSION_NAME=_C", f"-D_GLIBCXX_USE_CXX11_ABI={abi}",
+    defs = ["-DTORCH_API_INCLUDE_EXTENSION_H", f"-DTORCH_EXTENSION_NAME={name}", f"-D_GLIBCXX_USE_CXX11_ABI={abi}",
             "-DUSE_ROCM=1", "-D__HIP_PLATFORM_AMD__=1"]
     libdir = os.path.join(os.path.dirname(torch.__file__), "lib")
     libs = [f"-L{libdir}", f"-Wl,-rpath,{libdir}", "-lc10", "-ltorch", "-ltorch_cpu", "-ltorch_python",
@@ -78,24 +81,36 @@ def build_rt(force: bool = False) -> str:
 
 
 def build_C(force: bool = False, jobs: int = 8) -> str:
-    out = os.path.join(ROOT, "mxserve", "_C" + _ext_suffix())
-    kdir = os.path.join(ROOT, "csrc", "kernels")
-    headers = glob.glob(os.path.join(kdir, "*.h"))
+    return _build_torch_ext("_C", os.path.join(ROOT, "csrc", "kernels"), [], force, jobs)
+
+
+def build_M(force: bool = False, jobs: int = 8) -> str:
+    """The mixer kernels (csrc/mixers); they share csrc/kernels/common.h."""
+    return _build_torch_ext("_M", os.path.join(ROOT, "csrc", "mixers"),
+                            [os.path.join(ROOT, "csrc", "kernels", "common.h")], force, jobs)
+
+
+def _build_torch_ext(name: str, kdir: str, more_headers: list, force: bool, jobs: int) -> str:
+    out = os.path.join(ROOT, "mxserve", name + _ext_suffix())
+    headers = glob.glob(os.path.join(kdir, "*.h")) + more_headers
     hip_srcs = sorted(glob.glob(os.path.join(kdir, "*.hip")))
     cpp_srcs = sorted(glob.glob(os.path.join(kdir, "*.cpp")))
     os.makedirs(BUILD, exist_ok=True)
-    inc, defs, libs = _torch_flags()
+    inc, defs, libs = _torch_flags(name)
     jobs_list = []
     objs = []
+    pre = "" if name == "_C" else name + "."
     for src in hip_srcs:
-        obj = os.path.join(BUILD, os.path.basename(src) + ".o")
+        obj = os.path.join(BUILD, pre + os.path.basename(src) + ".o")
         objs.append(obj)
         if force or _stale(obj, [src, *headers]):
             jobs_list.append([HIPCC, f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=fast",
+                              # no packed-fp32 instructions: hipcc otherwise forms them from plain float code
+                              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
                               "-munsafe-fp-atomics", *(["-DMXS_DEBUG_KERNELS"] if DEBUG_KERNELS else []),
                               "-c", src, "-o", obj])
     for src in cpp_srcs:
-        obj = os.path.join(BUILD, os.path.basename(src) + ".o")
+        obj = os.path.join(BUILD, pre + os.path.basename(src) + ".o")
         objs.append(obj)
         if force or _stale(obj, [src, *headers]):
             jobs_list.append(["g++", "-O2", "-std=c++17", "-fPIC", f"-I{ROCM}/include", *inc, *defs,
@@ -113,7 +128,7 @@ def main(argv=None) -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--clean", action="store_true")
     ap.add_argument("-j", type=int, default=min(8, os.cpu_count() or 4))
-    ap.add_argument("--only", choices=["rt", "C"], default=None)
+    ap.add_argument("--only", choices=["rt", "C", "M"], default=None)
     a = ap.parse_args(argv)
     if a.only in (None, "rt"):
         print("[mxserve] building host runtime _rt", flush=True)
@@ -121,6 +136,9 @@ def main(argv=None) -> None:
     if a.only in (None, "C"):
         print(f"[mxserve] building HIP kernels _C for {ARCH}", flush=True)
         build_C(a.clean, a.j)
+    if a.only in (None, "M"):
+        print(f"[mxserve] building mixer kernels _M for {ARCH}", flush=True)
+        build_M(a.clean, a.j)
     print("[mxserve] build ok", flush=True)
 
 
