@@ -18,8 +18,8 @@ void launch_kv_write(void*, long, const void*, long, const void*, long, const in
 bool launch_window_attention(void*, const void*, long, const void*, long, const int*, int, const int*, const int*, int,
                              int, int, int, int, int, int, int, int, float, int, int, bool, hipStream_t);
 bool launch_matrix_scan(float*, const void*, long, const void*, long, const void*, long, const float*, const float*,
-                        float*, long, const int*, long, const int*, const int*, int, int, int, int, int, float, float,
-                        bool, bool, hipStream_t);
+                        float*, long, const int*, long, const int*, const int*, int, int, int, int, int, int, float,
+                        float, bool, bool, hipStream_t);
 }  // namespace mxs
 
 namespace {
@@ -184,8 +184,8 @@ void scan(bool mlstm, at::Tensor out, at::Tensor q, at::Tensor k, at::Tensor v, 
   const bool ok = mxs::launch_matrix_scan(
       op, mat(q, bf, T, H * dk, "q"), q.stride(0), mat(k, bf, T, H * dk, "k"), k.stride(0), mat(v, bf, T, H * dv, "v"),
       v.stride(0), decay, gates, sp, state.stride(0), i32(state_rows, S, "state_rows"), off, i32(qsl, S + 1, "qsl"),
-      i32(seq_lens, S, "seq_lens"), static_cast<int>(S), static_cast<int>(H), static_cast<int>(dk), static_cast<int>(dv),
-      silu ? 1 : 0, static_cast<float>(cap), static_cast<float>(q_scale), mlstm, bf, stream());
+      i32(seq_lens, S, "seq_lens"), static_cast<int>(S), static_cast<int>(T), static_cast<int>(H), static_cast<int>(dk),
+      static_cast<int>(dv), silu ? 1 : 0, static_cast<float>(cap), static_cast<float>(q_scale), mlstm, bf, stream());
   TORCH_CHECK(ok, "matrix scan: key size beyond 256");
 }
 

@@ -18,8 +18,8 @@ __global__ void __launch_bounds__(256) matrix_scan_kernel(
     float* __restrict__ out, const T* __restrict__ q, long q_stride, const T* __restrict__ k, long k_stride,
     const T* __restrict__ v, long v_stride, const float* __restrict__ decay, const float* __restrict__ gates,
     float* __restrict__ state, long state_stride, const int* __restrict__ state_rows, long off,
-    const int* __restrict__ qsl, const int* __restrict__ seq_lens, int H, int dk, int dv, int silu, float gate_cap,
-    float q_scale) {
+    const int* __restrict__ qsl, const int* __restrict__ seq_lens, int n_rows, int H, int dk, int dv, int silu,
+    float gate_cap, float q_scale) {
   constexpr int DT = 4 * DR;  // padded key size
   __shared__ float sk[kTB][DT];
   __shared__ float sq[kTB][DT];
@@ -29,7 +29,9 @@ __global__ void __launch_bounds__(256) matrix_scan_kernel(
   __shared__ float sfa[kTB], sia[kTB], sem[kTB];
   const int s = blockIdx.x, hd = blockIdx.y, c0 = blockIdx.z * 64;
   const int tid = threadIdx.x, j = tid & 63, r = tid >> 6;
-  const int row0 = qsl[s], qlen = qsl[s + 1] - row0;
+  const int row0 = qsl[s];
+  if (row0 < 0 || row0 >= n_rows) return;
+  const int qlen = min(qsl[s + 1], n_rows) - row0;  // never past the step's rows, whatever the metadata says
   if (qlen <= 0) return;
   const bool fresh = seq_lens[s] - qlen == 0;  // the sequence's first tokens: zero state
   const int col = c0 + j;
@@ -135,12 +137,12 @@ __global__ void __launch_bounds__(256) matrix_scan_kernel(
 template <typename T, bool MLSTM>
 static bool launch_scan_t(float* out, const T* q, long qs, const T* k, long ks, const T* v, long vs, const float* decay,
                           const float* gates, float* state, long state_stride, const int* state_rows, long off,
-                          const int* qsl, const int* seq_lens, int S, int H, int dk, int dv, int silu, float cap,
+                          const int* qsl, const int* seq_lens, int S, int n_rows, int H, int dk, int dv, int silu, float cap,
                           float q_scale, hipStream_t st) {
   const dim3 grid(S, H, (dv + 63) / 64), block(256);
 #define MIX_SCAN(DR)                                                                                               \
   hipLaunchKernelGGL((matrix_scan_kernel<T, DR, MLSTM>), grid, block, 0, st, out, q, qs, k, ks, v, vs, decay, gates, \
-                     state, state_stride, state_rows, off, qsl, seq_lens, H, dk, dv, silu, cap, q_scale)
+                     state, state_stride, state_rows, off, qsl, seq_lens, n_rows, H, dk, dv, silu, cap, q_scale)
   if (dk <= 32) MIX_SCAN(8);
   else if (dk <= 64) MIX_SCAN(16);
   else if (dk <= 128) MIX_SCAN(32);
@@ -153,21 +155,21 @@ static bool launch_scan_t(float* out, const T* q, long qs, const T* k, long ks, 
 
 bool launch_matrix_scan(float* out, const void* q, long qs, const void* k, long ks, const void* v, long vs,
                         const float* decay, const float* gates, float* state, long state_stride, const int* state_rows,
-                        long off, const int* qsl, const int* seq_lens, int S, int H, int dk, int dv, int silu, float cap,
-                        float q_scale, bool mlstm, bool bf, hipStream_t st) {
+                        long off, const int* qsl, const int* seq_lens, int S, int n_rows, int H, int dk, int dv, int silu,
+                        float cap, float q_scale, bool mlstm, bool bf, hipStream_t st) {
   if (S == 0) return true;
   if (bf) {
     using T = bf16_t;
     return mlstm ? launch_scan_t<T, true>(out, (const T*)q, qs, (const T*)k, ks, (const T*)v, vs, decay, gates, state,
-                                          state_stride, state_rows, off, qsl, seq_lens, S, H, dk, dv, silu, cap, q_scale, st)
+                                          state_stride, state_rows, off, qsl, seq_lens, S, n_rows, H, dk, dv, silu, cap, q_scale, st)
                  : launch_scan_t<T, false>(out, (const T*)q, qs, (const T*)k, ks, (const T*)v, vs, decay, gates, state,
-                                           state_stride, state_rows, off, qsl, seq_lens, S, H, dk, dv, silu, cap, q_scale, st);
+                                           state_stride, state_rows, off, qsl, seq_lens, S, n_rows, H, dk, dv, silu, cap, q_scale, st);
   }
   using T = float;
   return mlstm ? launch_scan_t<T, true>(out, (const T*)q, qs, (const T*)k, ks, (const T*)v, vs, decay, gates, state,
-                                        state_stride, state_rows, off, qsl, seq_lens, S, H, dk, dv, silu, cap, q_scale, st)
+                                        state_stride, state_rows, off, qsl, seq_lens, S, n_rows, H, dk, dv, silu, cap, q_scale, st)
                : launch_scan_t<T, false>(out, (const T*)q, qs, (const T*)k, ks, (const T*)v, vs, decay, gates, state,
-                                         state_stride, state_rows, off, qsl, seq_lens, S, H, dk, dv, silu, cap, q_scale, st);
+                                         state_stride, state_rows, off, qsl, seq_lens, S, n_rows, H, dk, dv, silu, cap, q_scale, st);
 }
 
 }  // namespace mxs

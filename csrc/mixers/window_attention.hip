@@ -26,7 +26,8 @@ __global__ void __launch_bounds__(256) window_attention_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
   const int s = seq_of_row(qsl, S, t);
   const int qlen = qsl[s + 1] - qsl[s];
-  const int pos = seq_lens[s] - qlen + (t - qsl[s]);
+  // the row's position, kept inside the block table whatever the metadata says
+  const int pos = min(max(seq_lens[s] - qlen + (t - qsl[s]), 0), bt_stride * bs - 1);
   const int g = hd / (H / G);
   const int lo = window > 0 ? max(pos - window + 1, 0) : 0;
   const int nA = window > 0 ? min(keep, lo) : 0;  // kept first tokens that lie below the window

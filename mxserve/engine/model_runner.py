@@ -346,6 +346,7 @@ class ModelRunner:
             h["positions"][S:graph_bs] = 0
             h["slot_mapping"][S:graph_bs] = -1
             h["seq_lens"][S:graph_bs] = 1
+            h["qsl"][S + 1:graph_bs + 1] = np.arange(S + 1, graph_bs + 1)  # one row each (a chunk step leaves other values)
             h["rows"][S:graph_bs] = self.pad_row
             h["srows"][S:graph_bs] = self.pad_row
             h["trow"][S:graph_bs] = self.pad_row

@@ -82,6 +82,17 @@ class DecayLinearAttention(Mixer):
         self.state_floats = heads * dim * vdim
         self._decay_dev: dict = {}
 
+    def decay_on(self, device) -> torch.Tensor:
+        """The per-head decays as an fp32 device tensor (made when the weights are loaded, so that no
+        host-to-device copy falls into a graph capture)."""
+        a = self._decay_dev.get(device)
+        if a is None:
+            a = self._decay_dev[device] = torch.tensor(self.decay, dtype=torch.float32, device=device)
+        return a
+
+    def finish_weights(self, w: dict) -> None:
+        self.decay_on(w[self.p + "o"].device)
+
     def proj_rows(self) -> list:
         n, m = self.heads * self.qk, self.heads * self.vd
         return [(self.p + "q", n), (self.p + "k", n), (self.p + "v", m), (self.p + "g", m)]
@@ -92,9 +103,7 @@ class DecayLinearAttention(Mixer):
     def forward(self, parts: list, h: torch.Tensor, w: dict, ctx: StepContext, koff: int, voff: int, soff: int):
         q, k, v, g = parts
         md = ctx.md
-        a = self._decay_dev.get(h.device)
-        if a is None:
-            a = self._decay_dev[h.device] = torch.tensor(self.decay, dtype=torch.float32, device=h.device)
+        a = self.decay_on(h.device)
         o = seqmix.decay_scan(q, k, v, a, ctx.state, md.state_rows, soff, md.query_start_loc, md.seq_lens,
                               self.heads, self.qk, self.vd, silu=True)
         y = seqmix.gated_rms_norm(o, g, w[self.p + "norm"], ctx.eps, 1, h.dtype)
