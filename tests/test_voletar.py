@@ -180,7 +180,8 @@ def test_mixed_batches_reuse_pages_and_slots(base, dev, dtype, tol, eager):
             steps.append(step)
     got = replay(eng, steps)
     for r in toks:  # bf16: a sequence's very first tokens round coarsely (one key, near-ties in the mLSTM's max)
-        _check(got[r][8:], want[r][8:], tol)
+        if len(toks[r]) > 8:
+            _check(got[r][8:], want[r][8:], tol)
         _check(got[r][:8], want[r][:8], tol if dtype == "float32" else 0.6)
     assert eng.kv.num_free() == eng.kv.num_blocks and not eng.runner._row_of
 
