@@ -99,6 +99,15 @@ def vlog(msg: str) -> None:
 def parse(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
+    # a separate measurement, not the headline: Voletar beside a Llama-shaped model of equal size
+    # (mxserve/tools/mixer_bench.py); without this flag nothing of the default workload changes
+    ap.add_argument("--mixer-bench", action="store_true",
+                    help="prefill / decode throughput of Voletar beside a Llama-shaped model of equal size, and the "
+                         "mixer kernels against their rooflines; prints JSON lines and exits")
+    ap.add_argument("--mixer-sizes", default="1024,2048", help="model widths, comma-separated")
+    ap.add_argument("--mixer-prompt", type=int, default=4096)
+    ap.add_argument("--mixer-batch", type=int, default=64)
+    ap.add_argument("--mixer-context", type=int, default=2048)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--iters-per-step", type=int, default=int(os.environ.get("MXS_BENCH_ITERS_PER_STEP", "50")),
@@ -1008,6 +1017,9 @@ def phase_disagg(a, ctx) -> tuple:
 
 def main():
     a = parse()
+    if a.mixer_bench:
+        from mxserve.tools.mixer_bench import main as mixer_main
+        return mixer_main([int(x) for x in a.mixer_sizes.split(",")], a.mixer_prompt, a.mixer_batch, a.mixer_context)
     world_env = os.environ.get("WORLD_SIZE")
     if world_env is None and a.gpus > 1:
         return launch_ranks(a)

@@ -42,7 +42,11 @@ void launch_ep_segment_rows(int*, const int*, int, int, hipStream_t);
 namespace {
 
 void hip_check(hipError_t e, const char* what) {
-  if (e != hipSuccess) throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
+  if (e == hipSuccess) return;
+  // a failed call also leaves its code as the runtime's "last error"; unread, the next kernel launch
+  // check anywhere in the process (torch's included) would report it as its own
+  (void)hipGetLastError();
+  throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
 }
 
 pybind11::tuple export_pool(at::Tensor t) {

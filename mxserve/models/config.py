@@ -184,6 +184,25 @@ def voletar_config(name: str, d: dict) -> ModelConfig:
         chat_template="chatml", arch_config=keep)
 
 
+# A small Voletar (random weights) with every kind of layer and a looped span, for tests and smoke runs.
+_reg(voletar_config("tiny-voletar", {
+    "architecture": "Voletar", "width": 128, "vocab": 512, "norm": {"eps": 1e-5}, "logit_softcap": 25.0,
+    "loop": {"start": 1, "stop": 3, "times": 2},
+    "layers": [
+        {"type": "lightning", "mlp": None,
+         "mixer": {"heads": 2, "dim": 32, "vdim": 64, "decay": [0.9, 0.99]}},
+        {"type": "parallel", "mlp": {"kind": "dense", "ff": 256},
+         "mixer": {"left": {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 48, "scale": 0.18,
+                            "mask": {"size": 40, "keep_first": 3}},
+                   "right": {"heads": 2, "dim": 16, "vdim": 32, "gate_cap": 10.0}}},
+        {"type": "lightning", "mlp": {"kind": "dense", "ff": 192},
+         "mixer": {"heads": 4, "dim": 16, "vdim": 16, "decay": [0.7, 0.9, 0.97, 0.995]}},
+        {"type": "parallel", "mlp": None,
+         "mixer": {"left": {"heads": 2, "kv_heads": 2, "dim": 64, "vdim": 64, "scale": 0.125,
+                            "mask": {"size": 16, "keep_first": 0}},
+                   "right": {"heads": 4, "dim": 32, "vdim": 16, "gate_cap": 8.0}}}]}))
+
+
 def _from_hf_json(name: str, d: dict) -> ModelConfig:
     if d.get("architecture") == "Voletar":
         return voletar_config(name, d)

@@ -1,0 +1,170 @@
+"""Prefill and decode throughput of Voletar beside a Llama-shaped model of equal width, depth and
+feed-forward size (random weights), through the same engine path: forced steps of the scheduler,
+the model runner, paged K/V and state slots, decode through the captured graphs.
+
+  python bench.py --mixer-bench [--mixer-sizes 1024,2048] [--mixer-prompt 4096] [--mixer-batch 64]
+
+Prints one JSON line per (size, model): prefill tokens/s of one prompt in one step, decode tokens/s
+of a batch of sequences at that context, and per-kernel times of the mixers against their
+roofline (FLOP and byte counts are the algorithm's own, stated next to each entry)."""
+from __future__ import annotations
+
+import dataclasses
+import json
+import time
+
+import torch
+
+from ..config import EngineArgs
+from ..engine.engine import LLMEngine
+from ..engine.replay import TraceReplayer
+from ..models import config as mcfg
+
+PEAK_BF16 = 2.5e15  # dense MFMA bf16 FLOP/s
+PEAK_F32 = 157e12  # VALU / fp32 MFMA FLOP/s
+PEAK_HBM = 8e12  # bytes/s
+
+
+def voletar_shape(width: int, layers: int = 4, window: int = 1024) -> dict:
+    """Alternating parallel / lightning layers with the head sizes of a model of this width."""
+    heads = width // 128
+    par = {"type": "parallel",
+           "mixer": {"left": {"heads": heads * 2, "kv_heads": max(heads // 2, 1), "dim": 64, "vdim": 64, "scale": 0.125,
+                              "mask": {"size": window, "keep_first": 4}},
+                     "right": {"heads": max(heads // 2, 1), "dim": 64, "vdim": 128, "gate_cap": 15.0}},
+           "mlp": {"kind": "dense", "ff": 4 * width}}
+    lig = {"type": "lightning", "mixer": {"heads": heads, "dim": 128, "vdim": 128,
+                                          "decay": [1.0 - 2.0 ** -(3 + 5 * i / max(heads - 1, 1)) for i in range(heads)]},
+           "mlp": {"kind": "dense", "ff": 4 * width}}
+    return {"architecture": "Voletar", "width": width, "vocab": 32000, "norm": {"eps": 1e-5}, "logit_softcap": 30.0,
+            "layers": [par if i % 2 == 0 else lig for i in range(layers)]}
+
+
+def register(width: int, layers: int) -> tuple:
+    v = mcfg.voletar_config(f"voletar-w{width}", voletar_shape(width, layers))
+    mcfg.REGISTRY[v.name.lower()] = v
+    base = mcfg.REGISTRY["small-llama"]
+    # gated feed-forward of 8/3 width has the parameters of a dense one of 4 width
+    l = dataclasses.replace(base, name=f"llama-w{width}", hidden_size=width, intermediate_size=(8 * width // 3) // 256 * 256,
+                            num_layers=layers, num_heads=width // 64, num_kv_heads=max(width // 256, 1), head_dim=64,
+                            vocab_size=32000, tie_word_embeddings=False)
+    mcfg.REGISTRY[l.name.lower()] = l
+    return v.name, l.name
+
+
+def _time(fn, reps: int) -> float:
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / reps
+
+
+def run_model(name: str, prompt: int, batch: int, context: int, reps: int = 5) -> dict:
+    bs = 16
+    blocks = (batch * (context + 64) + prompt) // bs + batch + 8
+    args = EngineArgs(model=name, device="cuda", dtype="bfloat16", block_size=bs, num_gpu_blocks=blocks,
+                      max_model_len=max(prompt, context) + 128, max_num_seqs=batch, max_num_batched_tokens=max(prompt, batch * 64),
+                      enable_prefix_caching=False, async_scheduling=False, load_format="random", cuda_graph_max_bs=batch)
+    eng = LLMEngine(args)
+    rp = TraceReplayer(eng)
+    g = torch.Generator().manual_seed(0)
+    V = eng.model_config.vocab_size
+    toks = lambda n: torch.randint(3, V, (n,), generator=g).tolist()  # noqa: E731
+    n_pf = [0]
+
+    def prefill():
+        n_pf[0] += 1
+        rid = f"p{n_pf[0]}"
+        rp.step([{"id": rid, "tokens": toks(prompt), "want": [prompt - 1]}], [rid])
+    prefill()
+    t_pf = _time(prefill, reps)
+    # decode: `batch` sequences brought to `context` tokens in chunks, then single tokens through the graphs
+    ids = [f"d{i}" for i in range(batch)]
+    per = max(1, min(batch, args.max_num_batched_tokens // context))
+    for i in range(0, batch, per):
+        rp.step([{"id": r, "tokens": toks(context), "want": []} for r in ids[i:i + per]], [])
+
+    def decode():
+        rp.step([{"id": r, "tokens": toks(1), "want": [0]} for r in ids], [])
+    decode()
+    t_dec = _time(decode, 4 * reps)
+    out = {"model": name, "params_m": round(eng.model_config.num_params() / 1e6, 1), "prompt": prompt,
+           "prefill_tok_s": round(prompt / t_pf), "prefill_ms": round(1e3 * t_pf, 3), "decode_batch": batch,
+           "decode_context": context, "decode_tok_s": round(batch / t_dec), "decode_step_ms": round(1e3 * t_dec, 3),
+           "decode_graph": bool(eng.runner.graphs)}
+    rp.step([], ids)
+    eng.close()
+    return out
+
+
+def kernel_rooflines(width: int, prompt: int, batch: int, context: int) -> list:
+    """The mixers' own kernels alone, at this size: time, and time over the roofline time."""
+    from .. import ops
+    from ..ops import seqmix
+    dev = torch.device("cuda")
+    dt = torch.bfloat16
+    bs, out = 16, []
+    heads = width // 128
+    i32 = dict(dtype=torch.int32, device=dev)
+
+    def entry(name, t, flops, peak, bytes_, note):
+        roof = max(flops / peak, bytes_ / PEAK_HBM)
+        out.append({"kernel": name, "width": width, "ms": round(1e3 * t, 4), "roofline_ms": round(1e3 * roof, 4),
+                    "x_roofline": round(t / roof, 1), "counts": note})
+
+    for mode, T, S, ctx in (("prefill", prompt, 1, prompt), ("decode", batch, batch, context)):
+        qsl = torch.arange(0, T + 1, T // S, **i32)
+        seq = torch.full((S,), ctx, **i32)
+        nb = -(-ctx // bs)
+        bt = torch.arange(S * nb, **i32).view(S, nb)
+        # window attention of the parallel layers
+        H, G, dk, dv, win = heads * 2, max(heads // 2, 1), 64, 64, 1024
+        cache = torch.randn(S * nb, G * bs * (dk + dv), device=dev).to(dt)
+        q = torch.randn(T, H * dk, device=dev).to(dt)
+        t = _time(lambda: seqmix.window_attention(q, cache, bt, qsl, seq, 0, G * bs * dk, H, G, dk, dv, bs, 0.125, win, 4), 5)
+        keys = min(win, ctx) if mode == "decode" else min(win, ctx / 2)
+        entry(f"window_attention/{mode}", t, 2.0 * T * H * keys * (dk + dv), PEAK_BF16,
+              2.0 * (S * min(win, ctx) * G * (dk + dv) + 2 * T * H * dk), f"{T} rows x {H} heads x ~{int(keys)} keys, bf16 MFMA peak")
+        # the closest kernel of the Llama path at the same head layout, full causal
+        kv = torch.randn(S * nb, 1, 2, G, bs, 64, device=dev).to(dt)
+        q3 = q.view(T, H, dk)
+        if mode == "prefill":
+            fn = lambda: ops.paged_attention_prefill(q3, kv[:, 0], bt, qsl, seq, 0.125, T)  # noqa: E731
+            keys_l = ctx / 2
+        else:
+            fn = lambda: ops.paged_attention_decode(q3, kv[:, 0], bt, seq, 0.125, ctx)  # noqa: E731
+            keys_l = ctx
+        t = _time(fn, 5)
+        entry(f"paged_attention/{mode} (llama)", t, 2.0 * T * H * keys_l * 128, PEAK_BF16,
+              2.0 * (S * ctx * G * 128 + 2 * T * H * dk), f"{T} rows x {H} heads x ~{int(keys_l)} keys, bf16 MFMA peak")
+        # the recurrences: fp32 state, two multiply-adds per state element and token
+        for name, Hh, d1, d2, mlstm in (("decay_scan", heads, 128, 128, False), ("mlstm_scan", max(heads // 2, 1), 64, 128, True)):
+            n = Hh * d1 * d2 + (Hh * (d1 + 1) if mlstm else 0)
+            state = torch.zeros(S, n, device=dev)
+            rows = torch.arange(S, **i32)
+            qq, kk = (torch.randn(T, Hh * d1, device=dev).to(dt) for _ in range(2))
+            vv = torch.randn(T, Hh * d2, device=dev).to(dt)
+            if mlstm:
+                gates = torch.randn(T, 2 * Hh, device=dev)
+                fn = lambda: seqmix.mlstm_scan(qq, kk, vv, gates, state, rows, 0, qsl, seq, Hh, d1, d2, 15.0, d1 ** -0.5)  # noqa: E731
+            else:
+                dec = torch.full((Hh,), 0.99, device=dev)
+                fn = lambda: seqmix.decay_scan(qq, kk, vv, dec, state, rows, 0, qsl, seq, Hh, d1, d2)  # noqa: E731
+            t = _time(fn, 5)
+            entry(f"{name}/{mode}", t, 4.0 * T * Hh * d1 * d2, PEAK_F32, 8.0 * S * n + 2.0 * T * Hh * (2 * d1 + 3 * d2),
+                  f"{T} rows x {Hh} heads x {d1}x{d2} state, fp32 peak; state read and written once")
+    return out
+
+
+def main(sizes: list, prompt: int, batch: int, context: int, layers: int = 4) -> int:
+    from .. import ops
+    ops.ext()
+    for width in sizes:
+        v, l = register(width, layers)
+        for name in (v, l):
+            print(json.dumps(run_model(name, prompt, batch, context)), flush=True)
+        for e in kernel_rooflines(width, prompt, batch, context):
+            print(json.dumps(e), flush=True)
+    return 0

@@ -31,8 +31,8 @@ def _manifests(base):
 
 @pytest.mark.parametrize("base", [ROOT, REF])
 def test_every_example_manifest_parses(base):
-    if not os.path.isdir(base):
-        pytest.skip("reference not mounted")
+    if not os.path.isdir(os.path.join(base, "examples")):
+        pytest.skip("reference not mounted (or mounted empty)")
     ms = _manifests(base)
     assert ms
     for path, d in ms:
@@ -497,8 +497,8 @@ def test_reference_manifests_deploy_unmodified(cluster, tmp_path, monkeypatch):
     /workspace working dirs, TRT-LLM engine YAMLs relative to /workspace), reconcile into pods that
     all run the mxserve image; each rewrite is recorded in the DCD status, and the engine YAML paths
     resolve inside the image layout."""
-    if not os.path.isdir(REF):
-        pytest.skip("reference not mounted")
+    if not os.path.isdir(os.path.join(REF, "examples")):
+        pytest.skip("reference not mounted (or mounted empty)")
     from mxserve.k8s.resources import DEFAULT_IMAGE
     from mxserve.worker.args import parse_worker_args, resolve_engine_args_path
     fake, k = cluster
