@@ -16,7 +16,7 @@ void launch_gate_linear(float*, const void*, long, const void*, const void*, int
 void launch_kv_write(void*, long, const void*, long, const void*, long, const int64_t*, int, int, int, int, int, int,
                      int, bool, hipStream_t);
 bool launch_window_attention(void*, const void*, long, const void*, long, const int*, int, const int*, const int*, int,
-                             int, int, int, int, int, int, int, int, float, int, int, bool, hipStream_t);
+                             int, int, int, int, int, int, int, int, float, int, int, int, bool, hipStream_t);
 bool launch_matrix_scan(float*, const void*, long, const void*, long, const void*, long, const float*, const float*,
                         float*, long, const int*, long, const int*, const int*, int, int, int, int, int, int, float,
                         float, bool, bool, hipStream_t);
@@ -153,7 +153,7 @@ void kv_write(at::Tensor cache, at::Tensor k, at::Tensor v, at::Tensor slots, in
 
 void window_attention(at::Tensor out, at::Tensor q, at::Tensor cache, at::Tensor block_tables, at::Tensor qsl,
                       at::Tensor seq_lens, int64_t koff, int64_t voff, int64_t H, int64_t G, int64_t dk, int64_t dv,
-                      int64_t bs, double scale, int64_t window, int64_t keep) {
+                      int64_t bs, double scale, int64_t window, int64_t keep, int64_t max_query_len) {
   const bool bf = is_bf(q);
   const int64_t T = q.size(0), S = seq_lens.numel();
   check_cache(cache, bf, koff, voff, G, dk, dv, bs);
@@ -167,7 +167,8 @@ void window_attention(at::Tensor out, at::Tensor q, at::Tensor cache, at::Tensor
       block_tables.data_ptr<int>(), static_cast<int>(block_tables.stride(0)), i32(qsl, S + 1, "qsl"),
       i32(seq_lens, S, "seq_lens"), static_cast<int>(S), static_cast<int>(T), static_cast<int>(koff),
       static_cast<int>(voff), static_cast<int>(H), static_cast<int>(G), static_cast<int>(dk), static_cast<int>(dv),
-      static_cast<int>(bs), static_cast<float>(scale), static_cast<int>(window), static_cast<int>(keep), bf, stream());
+      static_cast<int>(bs), static_cast<float>(scale), static_cast<int>(window), static_cast<int>(keep),
+      static_cast<int>(std::min<int64_t>(max_query_len, T)), bf, stream());
   TORCH_CHECK(ok, "window_attention: head sizes beyond what the kernel holds (dv <= 512)");
 }
 

@@ -168,12 +168,14 @@ def window_attention(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.T
     """Softmax attention over the paged cache (this step's keys already written).  The query at
     position i sees key j <= i when i - j < window or j < keep_first (window <= 0: every j <= i).
     q [T, H*dk] (row-strided view) -> [T, H*dv] in q's dtype; scores and weights in fp32.
-    Query head h reads kv head h // (H / Hkv)."""
+    Query head h reads kv head h // (H / Hkv).  max_query_len: the longest chunk of the step (host
+    int); from 16 rows a bf16 step with head sizes that are multiples of 16 runs the MFMA kernel."""
     T = q.shape[0]
     if _gpu(q):
         out = torch.empty(T, num_heads * dv, dtype=q.dtype, device=q.device)
         ext().window_attention(out, q, cache, block_tables, qsl, seq_lens, int(koff), int(voff), num_heads,
-                               num_kv_heads, dk, dv, block_size, float(scale), int(window), int(keep_first))
+                               num_kv_heads, dk, dv, block_size, float(scale), int(window), int(keep_first),
+                               int(max_query_len))
         return out
     out = torch.zeros(T, num_heads, dv, dtype=torch.float32)
     kc = cache[:, koff:koff + num_kv_heads * block_size * dk].view(-1, num_kv_heads, block_size, dk)

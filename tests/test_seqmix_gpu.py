@@ -120,7 +120,7 @@ def test_window_attention_paged(gpu, dt, H, G, dk, dv, window, keep):
             seq = torch.tensor([a + b for a, b in zip(before, new)], dtype=torch.int32)
         T = sum(new)
         slots = _slots(bt, before, new, bs)
-        proj = torch.randn(T, H * dk + G * dk + G * dv + 5).to(dt)
+        proj = torch.randn(T, H * dk + G * dk + G * dv + 8).to(dt)
         q, k, v = proj[:, :H * dk], proj[:, H * dk:H * dk + G * dk], proj[:, H * dk + G * dk:H * dk + G * dk + G * dv]
         seqmix.kv_write(cache_c, k, v, slots, koff, voff, G, dk, dv, bs)
         pg = proj.to(gpu)
@@ -132,6 +132,10 @@ def test_window_attention_paged(gpu, dt, H, G, dk, dv, window, keep):
         og = seqmix.window_attention(qg, cache_g, bt.to(gpu), qsl.to(gpu), seq.to(gpu), koff, voff, H, G, dk, dv, bs, 0.13,
                                      window, keep)
         torch.testing.assert_close(og.cpu().float(), oc.float(), **_tol(dt))
+        # told the longest chunk, a bf16 step with MFMA-shaped heads takes the matrix-core kernel
+        om = seqmix.window_attention(qg, cache_g, bt.to(gpu), qsl.to(gpu), seq.to(gpu), koff, voff, H, G, dk, dv, bs, 0.13,
+                                     window, keep, max_query_len=max(new))
+        torch.testing.assert_close(om.cpu().float(), oc.float(), **_tol(dt))
 
 
 def test_kv_write_skips_padding(gpu):
