@@ -19,7 +19,7 @@ bool launch_window_attention(void*, const void*, long, const void*, long, const 
                              int, int, int, int, int, int, int, int, float, int, int, int, bool, hipStream_t);
 bool launch_matrix_scan(float*, const void*, long, const void*, long, const void*, long, const float*, const float*,
                         float*, long, const int*, long, const int*, const int*, int, int, int, int, int, int, float,
-                        float, bool, bool, hipStream_t);
+                        float, bool, bool, int, int, float*, float*, long, hipStream_t);
 }  // namespace mxs
 
 namespace {
@@ -174,7 +174,8 @@ void window_attention(at::Tensor out, at::Tensor q, at::Tensor cache, at::Tensor
 
 void scan(bool mlstm, at::Tensor out, at::Tensor q, at::Tensor k, at::Tensor v, const float* decay, const float* gates,
           at::Tensor state, at::Tensor state_rows, int64_t off, at::Tensor qsl, at::Tensor seq_lens, int64_t H,
-          int64_t dk, int64_t dv, bool silu, double cap, double q_scale) {
+          int64_t dk, int64_t dv, bool silu, double cap, double q_scale, int64_t piece, int64_t npieces, OptT sc_local,
+          OptT sc_start) {
   const bool bf = is_bf(q);
   const int64_t T = q.size(0), S = seq_lens.numel();
   float* op = f32(out, "out");
@@ -182,27 +183,42 @@ void scan(bool mlstm, at::Tensor out, at::Tensor q, at::Tensor k, at::Tensor v, 
   float* sp = f32(state, "state");
   const int64_t need = mlstm ? H * (dk * dv + dk + 1) : H * dk * dv;
   TORCH_CHECK(state.dim() == 2 && off >= 0 && off + need <= state.size(1), "state slot too small for this layer");
+  // time-split launches: two scratch pools of [S, npieces, sc_floats] (a piece's end state; mLSTM: plus [H] sums)
+  const int64_t sc_floats = need + (mlstm ? H : 0);
+  float *scl = nullptr, *scs = nullptr;
+  if (npieces > 1) {
+    TORCH_CHECK(piece >= 16 && sc_local.has_value() && sc_start.has_value(), "a split scan needs its scratch pools");
+    scl = f32(*sc_local, "sc_local");
+    scs = f32(*sc_start, "sc_start");
+    TORCH_CHECK(sc_local->numel() >= S * npieces * sc_floats && sc_start->numel() >= S * npieces * sc_floats,
+                "scratch pools smaller than [S, npieces, state]");
+  } else {
+    piece = 1;
+    npieces = 1;
+  }
   const bool ok = mxs::launch_matrix_scan(
       op, mat(q, bf, T, H * dk, "q"), q.stride(0), mat(k, bf, T, H * dk, "k"), k.stride(0), mat(v, bf, T, H * dv, "v"),
       v.stride(0), decay, gates, sp, state.stride(0), i32(state_rows, S, "state_rows"), off, i32(qsl, S + 1, "qsl"),
       i32(seq_lens, S, "seq_lens"), static_cast<int>(S), static_cast<int>(T), static_cast<int>(H), static_cast<int>(dk),
-      static_cast<int>(dv), silu ? 1 : 0, static_cast<float>(cap), static_cast<float>(q_scale), mlstm, bf, stream());
+      static_cast<int>(dv), silu ? 1 : 0, static_cast<float>(cap), static_cast<float>(q_scale), mlstm, bf,
+      static_cast<int>(piece), static_cast<int>(npieces), scl, scs, sc_floats, stream());
   TORCH_CHECK(ok, "matrix scan: key size beyond 256");
 }
 
 void decay_scan(at::Tensor out, at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor decay, at::Tensor state,
                 at::Tensor state_rows, int64_t off, at::Tensor qsl, at::Tensor seq_lens, int64_t H, int64_t dk,
-                int64_t dv, bool silu) {
+                int64_t dv, bool silu, int64_t piece, int64_t npieces, OptT sc_local, OptT sc_start) {
   TORCH_CHECK(decay.numel() == H, "decay: fp32 [H]");
-  scan(false, out, q, k, v, f32(decay, "decay"), nullptr, state, state_rows, off, qsl, seq_lens, H, dk, dv, silu, 0.0, 1.0);
+  scan(false, out, q, k, v, f32(decay, "decay"), nullptr, state, state_rows, off, qsl, seq_lens, H, dk, dv, silu, 0.0, 1.0,
+       piece, npieces, sc_local, sc_start);
 }
 
 void mlstm_scan(at::Tensor out, at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor gates, at::Tensor state,
                 at::Tensor state_rows, int64_t off, at::Tensor qsl, at::Tensor seq_lens, int64_t H, int64_t dk,
-                int64_t dv, double cap, double q_scale) {
+                int64_t dv, double cap, double q_scale, int64_t piece, int64_t npieces, OptT sc_local, OptT sc_start) {
   TORCH_CHECK(gates.dim() == 2 && gates.size(0) == q.size(0) && gates.size(1) == 2 * H, "gates: fp32 [T, 2H]");
   scan(true, out, q, k, v, nullptr, f32(gates, "gates"), state, state_rows, off, qsl, seq_lens, H, dk, dv, false, cap,
-       q_scale);
+       q_scale, piece, npieces, sc_local, sc_start);
 }
 
 }  // namespace

@@ -105,7 +105,7 @@ class DecayLinearAttention(Mixer):
         md = ctx.md
         a = self.decay_on(h.device)
         o = seqmix.decay_scan(q, k, v, a, ctx.state, md.state_rows, soff, md.query_start_loc, md.seq_lens,
-                              self.heads, self.qk, self.vd, silu=True)
+                              self.heads, self.qk, self.vd, silu=True, max_query_len=md.max_query_len)
         y = seqmix.gated_rms_norm(o, g, w[self.p + "norm"], ctx.eps, 1, h.dtype)
         return ops.linear(y, w[self.p + "o"])
 
@@ -137,7 +137,8 @@ class MLSTM(Mixer):
         md = ctx.md
         gates = seqmix.gate_linear(h, w[self.p + "_if"], w[self.p + "_if.b"])
         o = seqmix.mlstm_scan(q, k, v, gates, ctx.state, md.state_rows, soff, md.query_start_loc, md.seq_lens,
-                              self.heads, self.qk, self.vd, self.gate_cap, self.qk ** -0.5)
+                              self.heads, self.qk, self.vd, self.gate_cap, self.qk ** -0.5,
+                              max_query_len=md.max_query_len)
         y = seqmix.gated_rms_norm(o, g, w[self.p + "norm"], ctx.eps, self.heads, h.dtype)
         return ops.linear(y, w[self.p + "o"])
 

@@ -204,17 +204,37 @@ def window_attention(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.T
 
 
 # ----------------------------------------------------------------------------- recurrences
+SCAN_PIECE = 256  # tokens per piece of a time-split scan
+SCAN_SCRATCH_BYTES = 512 << 20
+
+
+def _scan_split(S: int, max_query_len: int, floats: int, device) -> tuple:
+    """(piece, npieces, scratch pool, scratch pool) of a scan launch: chunks of 2 pieces or more are cut
+    into pieces that run side by side (two passes and a chaining step, csrc/mixers/scan.hip); the
+    pieces grow until both scratch pools [S, npieces, state] fit SCAN_SCRATCH_BYTES."""
+    piece = SCAN_PIECE
+    while max_query_len >= 2 * piece:
+        n = -(-max_query_len // piece)
+        if 2 * S * n * floats * 4 <= SCAN_SCRATCH_BYTES:
+            pool = torch.empty(2, S * n * floats, dtype=torch.float32, device=device)
+            return piece, n, pool[0], pool[1]
+        piece *= 2
+    return 1, 1, None, None
+
+
 def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, state: torch.Tensor,
                state_rows: torch.Tensor, off: int, qsl: torch.Tensor, seq_lens: torch.Tensor, num_heads: int,
-               dk: int, dv: int, silu: bool = True) -> torch.Tensor:
+               dk: int, dv: int, silu: bool = True, max_query_len: int = 0) -> torch.Tensor:
     """Decayed linear attention, token by token per head: S = decay_h S + k v^T, o = S^T q, with q, k, v
     passed through SiLU first when `silu`.  q, k [T, H*dk], v [T, H*dv] (row-strided views); decay
-    fp32 [H]; returns o fp32 [T, H*dv] and leaves each sequence's S in its slot."""
+    fp32 [H]; returns o fp32 [T, H*dv] and leaves each sequence's S in its slot.  max_query_len: the
+    step's longest chunk (host int); long chunks are cut into pieces that run side by side."""
     T = q.shape[0]
     if _gpu(q):
         out = torch.empty(T, num_heads * dv, dtype=torch.float32, device=q.device)
+        plan = _scan_split(seq_lens.numel(), min(max_query_len, T), num_heads * dk * dv, q.device)
         ext().decay_scan(out, q, k, v, decay, state, state_rows, int(off), qsl, seq_lens, num_heads, dk, dv,
-                         bool(silu))
+                         bool(silu), *plan)
         return out
     out = torch.zeros(T, num_heads, dv, dtype=torch.float32)
     qf, kf, vf = (t.float().reshape(T, num_heads, -1) for t in (q, k, v))
@@ -241,7 +261,7 @@ def mlstm_state_floats(num_heads: int, dk: int, dv: int) -> int:
 
 def mlstm_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gates: torch.Tensor, state: torch.Tensor,
                state_rows: torch.Tensor, off: int, qsl: torch.Tensor, seq_lens: torch.Tensor, num_heads: int,
-               dk: int, dv: int, gate_cap: float, q_scale: float) -> torch.Tensor:
+               dk: int, dv: int, gate_cap: float, q_scale: float, max_query_len: int = 0) -> torch.Tensor:
     """mLSTM matrix memory, token by token per head.  gates fp32 [T, 2H]: the input gates' then the
     forget gates' pre-activations.  With i = cap tanh(pre_i / cap), f = logsigmoid(cap tanh(pre_f / cap))
     and a running maximum m (0 at the start):
@@ -251,8 +271,10 @@ def mlstm_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gates: torch.T
     T = q.shape[0]
     if _gpu(q):
         out = torch.empty(T, num_heads * dv, dtype=torch.float32, device=q.device)
+        plan = _scan_split(seq_lens.numel(), min(max_query_len, T), mlstm_state_floats(num_heads, dk, dv) + num_heads,
+                           q.device)
         ext().mlstm_scan(out, q, k, v, gates, state, state_rows, int(off), qsl, seq_lens, num_heads, dk, dv,
-                         float(gate_cap), float(q_scale))
+                         float(gate_cap), float(q_scale), *plan)
         return out
     H = num_heads
     out = torch.zeros(T, H, dv, dtype=torch.float32)

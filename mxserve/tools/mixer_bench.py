@@ -123,7 +123,8 @@ def kernel_rooflines(width: int, prompt: int, batch: int, context: int) -> list:
         H, G, dk, dv, win = heads * 2, max(heads // 2, 1), 64, 64, 1024
         cache = torch.randn(S * nb, G * bs * (dk + dv), device=dev).to(dt)
         q = torch.randn(T, H * dk, device=dev).to(dt)
-        t = _time(lambda: seqmix.window_attention(q, cache, bt, qsl, seq, 0, G * bs * dk, H, G, dk, dv, bs, 0.125, win, 4), 5)
+        t = _time(lambda: seqmix.window_attention(q, cache, bt, qsl, seq, 0, G * bs * dk, H, G, dk, dv, bs, 0.125, win, 4,
+                                                  max_query_len=T // S), 5)
         keys = min(win, ctx) if mode == "decode" else min(win, ctx / 2)
         entry(f"window_attention/{mode}", t, 2.0 * T * H * keys * (dk + dv), PEAK_BF16,
               2.0 * (S * min(win, ctx) * G * (dk + dv) + 2 * T * H * dk), f"{T} rows x {H} heads x ~{int(keys)} keys, bf16 MFMA peak")
@@ -148,10 +149,11 @@ def kernel_rooflines(width: int, prompt: int, batch: int, context: int) -> list:
             vv = torch.randn(T, Hh * d2, device=dev).to(dt)
             if mlstm:
                 gates = torch.randn(T, 2 * Hh, device=dev)
-                fn = lambda: seqmix.mlstm_scan(qq, kk, vv, gates, state, rows, 0, qsl, seq, Hh, d1, d2, 15.0, d1 ** -0.5)  # noqa: E731
+                fn = lambda: seqmix.mlstm_scan(qq, kk, vv, gates, state, rows, 0, qsl, seq, Hh, d1, d2, 15.0, d1 ** -0.5,  # noqa: E731
+                                               max_query_len=T // S)
             else:
                 dec = torch.full((Hh,), 0.99, device=dev)
-                fn = lambda: seqmix.decay_scan(qq, kk, vv, dec, state, rows, 0, qsl, seq, Hh, d1, d2)  # noqa: E731
+                fn = lambda: seqmix.decay_scan(qq, kk, vv, dec, state, rows, 0, qsl, seq, Hh, d1, d2, max_query_len=T // S)  # noqa: E731
             t = _time(fn, 5)
             entry(f"{name}/{mode}", t, 4.0 * T * Hh * d1 * d2, PEAK_F32, 8.0 * S * n + 2.0 * T * Hh * (2 * d1 + 3 * d2),
                   f"{T} rows x {Hh} heads x {d1}x{d2} state, fp32 peak; state read and written once")

@@ -177,3 +177,36 @@ def test_scans_chunked_with_slot_reuse(gpu, dt, H, dk, dv):
         live = sorted(set(rows))
         torch.testing.assert_close(st_g.cpu()[live, pad:pad + nl + nm], st_c[live, pad:pad + nl + nm], rtol=2e-4, atol=2e-4)
         assert torch.equal(st_g.cpu()[:, :pad], st_c[:, :pad]) and torch.equal(st_g.cpu()[:, pad + nl + nm:], st_c[:, pad + nl + nm:])
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,dk,dv", [(3, 40, 64), (2, 128, 72)])
+def test_scans_split_over_time(gpu, dt, H, dk, dv):
+    """Chunks of two pieces or more run as pieces side by side (end states chained): same outputs and
+    end state as the serial walk, for fresh and continued sequences, next to a single-token row."""
+    torch.manual_seed(6)
+    nl, nm = H * dk * dv, seqmix.mlstm_state_floats(H, dk, dv)
+    st_c = torch.randn(4, nl + nm)
+    st_g = st_c.to(gpu)
+    decay = torch.tensor([0.9, 0.99, 0.999][:H])
+    for before, new, rows in (([0, 0, 0], [700, 1, 1300], [3, 1, 0]), ([700, 1, 1300], [513, 1, 1], [3, 1, 0])):
+        T = sum(new)
+        qsl = torch.tensor([0] + list(torch.tensor(new).cumsum(0)), dtype=torch.int32)
+        seq = torch.tensor([a + b for a, b in zip(before, new)], dtype=torch.int32)
+        rows_t = torch.tensor(rows, dtype=torch.int32)
+        proj = (0.5 * torch.randn(T, 2 * H * dk + H * dv)).to(dt)
+        q, k, v = proj[:, :H * dk], proj[:, H * dk:2 * H * dk], proj[:, 2 * H * dk:]
+        gates = torch.randn(T, 2 * H) * 3 + torch.tensor([0.0] * H + [3.0] * H)
+        pg = proj.to(gpu)
+        qg, kg, vg = pg[:, :H * dk], pg[:, H * dk:2 * H * dk], pg[:, 2 * H * dk:]
+        mq = max(new)
+        oc = seqmix.decay_scan(q, k, v, decay, st_c, rows_t, 0, qsl, seq, H, dk, dv)
+        og = seqmix.decay_scan(qg, kg, vg, decay.to(gpu), st_g, rows_t.to(gpu), 0, qsl.to(gpu), seq.to(gpu), H, dk, dv,
+                               max_query_len=mq)
+        torch.testing.assert_close(og.cpu(), oc, rtol=5e-4, atol=5e-4)
+        oc = seqmix.mlstm_scan(q, k, v, gates, st_c, rows_t, nl, qsl, seq, H, dk, dv, 9.0, dk ** -0.5)
+        og = seqmix.mlstm_scan(qg, kg, vg, gates.to(gpu), st_g, rows_t.to(gpu), nl, qsl.to(gpu), seq.to(gpu), H, dk, dv, 9.0,
+                               dk ** -0.5, max_query_len=mq)
+        torch.testing.assert_close(og.cpu(), oc, rtol=5e-4, atol=5e-4)
+        live = sorted(set(rows))
+        torch.testing.assert_close(st_g.cpu()[live], st_c[live], rtol=5e-4, atol=5e-4)
