@@ -85,6 +85,132 @@ __global__ void __launch_bounds__(256) window_attention_kernel(
 }
 
 
+// ---- Row form with 16-byte loads (single decoded tokens, short chunks): head sizes that are
+// multiples of 16 bytes.  Eight lanes share a key: each loads 16 bytes of every 128-byte stretch of
+// the key's row, so a wave's load instruction covers eight whole rows instead of 64 two-byte (or 64
+// scattered 16-byte) pieces; the score is summed over the eight lanes.  The value rows are read the
+// same way with the weight of their key, and the 32 key slots of the block are summed at the end
+// (three lane exchanges, then the four waves through LDS).
+template <typename T> struct El;
+template <> struct El<bf16_t> { static constexpr int N = 8; };
+template <> struct El<float> { static constexpr int N = 4; };
+__device__ __forceinline__ void load16(const bf16_t* p, float* o) {
+  const uint4 a = *reinterpret_cast<const uint4*>(p);
+  o[0] = bf2f_lo(a.x); o[1] = bf2f_hi(a.x); o[2] = bf2f_lo(a.y); o[3] = bf2f_hi(a.y);
+  o[4] = bf2f_lo(a.z); o[5] = bf2f_hi(a.z); o[6] = bf2f_lo(a.w); o[7] = bf2f_hi(a.w);
+}
+__device__ __forceinline__ void load16(const float* p, float* o) {
+  const float4 a = *reinterpret_cast<const float4*>(p);
+  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+}
+
+template <typename T, int NC>  // NC: 128-byte stretches of a row (head sizes <= NC * 8 * El<T>::N)
+__global__ void __launch_bounds__(256) window_attention_rows_kernel(
+    T* __restrict__ out, const T* __restrict__ q, long q_stride, const T* __restrict__ cache, long block_stride,
+    const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ qsl, const int* __restrict__ seq_lens,
+    int S, int koff, int voff, int H, int G, int dk, int dv, int bs, float scale, int window, int keep) {
+  constexpr int EL = El<T>::N;
+  extern __shared__ float lds[];
+  float* p = lds;                // [kKeyTile]
+  float* red = p + kKeyTile;     // [4][dv]
+  __shared__ float scratch[16];
+  const int t = blockIdx.x, hd = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
+  const int part = tid & 7, slot = tid >> 3;  // the lane's 16 bytes of each stretch; its key slot (0..31)
+  const int s = seq_of_row(qsl, S, t);
+  const int qlen = qsl[s + 1] - qsl[s];
+  const int pos = min(max(seq_lens[s] - qlen + (t - qsl[s]), 0), bt_stride * bs - 1);
+  const int g = hd / (H / G);
+  const int lo = window > 0 ? max(pos - window + 1, 0) : 0;
+  const int nA = window > 0 ? min(keep, lo) : 0;
+  const int nvis = nA + (pos - lo + 1);
+  const int* bt = block_tables + static_cast<long>(s) * bt_stride;
+  float qf[NC][EL], acc[NC][EL];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int d = (c * 8 + part) * EL;
+#pragma unroll
+    for (int e = 0; e < EL; ++e) {
+      qf[c][e] = d + e < dk ? ldf(q + static_cast<long>(t) * q_stride + hd * dk + d + e) * scale : 0.f;
+      acc[c][e] = 0.f;
+    }
+  }
+  float m = -INFINITY, l = 0.f;
+  for (int t0 = 0; t0 < nvis; t0 += kKeyTile) {
+    const int nt = min(kKeyTile, nvis - t0);
+    for (int n = slot; n < nt; n += 32) {
+      const int nn = t0 + n;
+      const int j = nn < nA ? nn : lo + (nn - nA);
+      const T* kp = cache + static_cast<long>(bt[j / bs]) * block_stride + koff + (static_cast<long>(g) * bs + j % bs) * dk;
+      float sc = 0.f;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const int d = (c * 8 + part) * EL;
+        if (d < dk) {
+          float kf[EL];
+          load16(kp + d, kf);
+#pragma unroll
+          for (int e = 0; e < EL; ++e) sc += qf[c][e] * kf[e];
+        }
+      }
+      sc += __shfl_xor(sc, 1, 64);
+      sc += __shfl_xor(sc, 2, 64);
+      sc += __shfl_xor(sc, 4, 64);
+      if (part == 0) p[n] = sc;
+    }
+    __syncthreads();
+    const float sc = tid < nt ? p[tid] : -INFINITY;
+    const float m_new = fmaxf(m, block_max(sc, scratch));
+    const float e = tid < nt ? expf(sc - m_new) : 0.f;
+    __syncthreads();  // every score is read before it is replaced by its weight
+    p[tid] = e;
+    const float tsum = block_sum(e, scratch);  // its barriers also publish p
+    const float corr = expf(m - m_new);
+    l = l * corr + tsum;
+    m = m_new;
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+#pragma unroll
+      for (int e2 = 0; e2 < EL; ++e2) acc[c][e2] *= corr;
+    for (int n = slot; n < nt; n += 32) {
+      const int nn = t0 + n;
+      const int j = nn < nA ? nn : lo + (nn - nA);
+      const T* vp = cache + static_cast<long>(bt[j / bs]) * block_stride + voff + (static_cast<long>(g) * bs + j % bs) * dv;
+      const float pn = p[n];
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const int d = (c * 8 + part) * EL;
+        if (d < dv) {
+          float vf[EL];
+          load16(vp + d, vf);
+#pragma unroll
+          for (int e2 = 0; e2 < EL; ++e2) acc[c][e2] += pn * vf[e2];
+        }
+      }
+    }
+    __syncthreads();  // p is rewritten by the next tile
+  }
+  // the 8 key slots of a wave that share `part`, then the 4 waves
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+#pragma unroll
+    for (int e2 = 0; e2 < EL; ++e2) {
+      float v = acc[c][e2];
+      v += __shfl_xor(v, 8, 64);
+      v += __shfl_xor(v, 16, 64);
+      v += __shfl_xor(v, 32, 64);
+      const int d = (c * 8 + part) * EL + e2;
+      if (lane < 8 && d < dv) red[wid * dv + d] = v;
+    }
+  }
+  __syncthreads();
+  const float inv = 1.f / l;
+  for (int e2 = tid; e2 < dv; e2 += blockDim.x) {
+    const float o = red[e2] + red[dv + e2] + red[2 * dv + e2] + red[3 * dv + e2];
+    stf(out + static_cast<long>(t) * (H * dv) + hd * dv + e2, o * inv);
+  }
+}
+
 // ---- MFMA form for prompt chunks (bf16, 16-token cache blocks, head sizes multiples of 16 up to
 // 16 * KSM / 16 * VTM).  A wave owns 16 consecutive query rows of one head and walks the visible
 // cache blocks (the kept first blocks, then the window's); no LDS, no barriers.  Per block, with
@@ -228,6 +354,18 @@ bool launch_window_attention(void* out, const void* q, long q_stride, const void
   const bool vec = dk % el == 0 && koff % el == 0 && block_stride % el == 0;
   const size_t shm = (((dk + 3) & ~3) + kKeyTile + 4 * dv) * sizeof(float);
   if (shm > 60 * 1024) return false;
+  if (vec && dv % el == 0 && voff % el == 0 && dk <= 256 && dv <= 256) {  // rows of whole 16-byte pieces
+    if (bf)
+      hipLaunchKernelGGL((window_attention_rows_kernel<bf16_t, 4>), dim3(rows, H), dim3(256), shm, st, (bf16_t*)out,
+                         (const bf16_t*)q, q_stride, (const bf16_t*)cache, block_stride, block_tables, bt_stride, qsl,
+                         seq_lens, S, koff, voff, H, G, dk, dv, bs, scale, window, keep);
+    else
+      hipLaunchKernelGGL((window_attention_rows_kernel<float, 8>), dim3(rows, H), dim3(256), shm, st, (float*)out,
+                         (const float*)q, q_stride, (const float*)cache, block_stride, block_tables, bt_stride, qsl,
+                         seq_lens, S, koff, voff, H, G, dk, dv, bs, scale, window, keep);
+    MXS_CHECK_LAUNCH();
+    return true;
+  }
   if (bf)
     hipLaunchKernelGGL(window_attention_kernel<bf16_t>, dim3(rows, H), dim3(256), shm, st, (bf16_t*)out, (const bf16_t*)q,
                        q_stride, (const bf16_t*)cache, block_stride, block_tables, bt_stride, qsl, seq_lens, S, koff,

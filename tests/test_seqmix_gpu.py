@@ -90,7 +90,7 @@ def test_small_ops(gpu, dt):
 
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("H,G,dk,dv,window,keep", [(5, 5, 80, 96, 50, 12), (4, 2, 40, 72, 9, 3), (8, 2, 64, 128, 300, 0),
-                                                    (3, 1, 24, 200, 0, 0), (2, 2, 128, 64, 5, 11)])
+                                                    (3, 1, 24, 200, 0, 0), (2, 2, 128, 64, 5, 11), (2, 1, 10, 6, 30, 2), (4, 2, 20, 36, 7, 1)])
 def test_window_attention_paged(gpu, dt, H, G, dk, dv, window, keep):
     """Two rounds over the same pool: prompt chunks, then mixed single tokens and chunks."""
     torch.manual_seed(2)
