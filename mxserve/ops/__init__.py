@@ -24,7 +24,18 @@ def ext():
     global _EXT, _EXT_ERR
     if _EXT is None and _EXT_ERR is None:
         try:
-            _EXT = importlib.import_module("mxserve._C")
+            try:
+                _EXT = importlib.import_module("mxserve._C")
+            except ModuleNotFoundError:
+                # a fresh checkout: build it in-tree once (hipcc), as _native.rt() and seqmix.ext() do
+                import sys
+                root = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+                if root not in sys.path:
+                    sys.path.insert(0, root)
+                import setup_ext
+                setup_ext.build_C()
+                importlib.invalidate_caches()
+                _EXT = importlib.import_module("mxserve._C")
         except BaseException as e:  # noqa: BLE001 - re-raised on first GPU use
             _EXT_ERR = e
     if _EXT is None:
