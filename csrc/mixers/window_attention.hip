@@ -104,45 +104,56 @@ __device__ __forceinline__ void load16(const float* p, float* o) {
   o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
 }
 
-template <typename T, int NC>  // NC: 128-byte stretches of a row (head sizes <= NC * 8 * El<T>::N)
+// NC: 128-byte stretches of a row (head sizes <= NC * 8 * El<T>::N).  RM: query heads of one kv head that
+// a workgroup serves together: a key or value row is loaded once and used for all of them.
+template <typename T, int NC, int RM>
 __global__ void __launch_bounds__(256) window_attention_rows_kernel(
     T* __restrict__ out, const T* __restrict__ q, long q_stride, const T* __restrict__ cache, long block_stride,
     const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ qsl, const int* __restrict__ seq_lens,
-    int S, int koff, int voff, int H, int G, int dk, int dv, int bs, float scale, int window, int keep) {
+    int S, int koff, int voff, int H, int G, int dk, int dv, int bs, float scale, int window, int keep, int nsplit) {
   constexpr int EL = El<T>::N;
   extern __shared__ float lds[];
-  float* p = lds;                // [kKeyTile]
-  float* red = p + kKeyTile;     // [4][dv]
-  __shared__ float scratch[16];
-  const int t = blockIdx.x, hd = blockIdx.y;
+  float* p = lds;                      // [RM][kKeyTile]
+  float* red = p + RM * kKeyTile;      // [4][RM][dv]
+  __shared__ float scratch[RM * 4];
+  const int t = blockIdx.x;
+  const int g = blockIdx.y / nsplit, hs = blockIdx.y - g * nsplit;
+  const int R = H / G;
+  const int h0 = g * R + hs * RM;      // first query head of this workgroup
+  const int nr = min(RM, R - hs * RM);
   const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
   const int part = tid & 7, slot = tid >> 3;  // the lane's 16 bytes of each stretch; its key slot (0..31)
   const int s = seq_of_row(qsl, S, t);
   const int qlen = qsl[s + 1] - qsl[s];
   const int pos = min(max(seq_lens[s] - qlen + (t - qsl[s]), 0), bt_stride * bs - 1);
-  const int g = hd / (H / G);
   const int lo = window > 0 ? max(pos - window + 1, 0) : 0;
   const int nA = window > 0 ? min(keep, lo) : 0;
   const int nvis = nA + (pos - lo + 1);
   const int* bt = block_tables + static_cast<long>(s) * bt_stride;
-  float qf[NC][EL], acc[NC][EL];
+  float qf[RM][NC][EL], acc[RM][NC][EL], m[RM], l[RM];
 #pragma unroll
-  for (int c = 0; c < NC; ++c) {
-    const int d = (c * 8 + part) * EL;
+  for (int r = 0; r < RM; ++r) {
+    m[r] = -INFINITY;
+    l[r] = 0.f;
 #pragma unroll
-    for (int e = 0; e < EL; ++e) {
-      qf[c][e] = d + e < dk ? ldf(q + static_cast<long>(t) * q_stride + hd * dk + d + e) * scale : 0.f;
-      acc[c][e] = 0.f;
+    for (int c = 0; c < NC; ++c) {
+      const int d = (c * 8 + part) * EL;
+#pragma unroll
+      for (int e = 0; e < EL; ++e) {
+        qf[r][c][e] = (r < nr && d + e < dk) ? ldf(q + static_cast<long>(t) * q_stride + (h0 + r) * dk + d + e) * scale : 0.f;
+        acc[r][c][e] = 0.f;
+      }
     }
   }
-  float m = -INFINITY, l = 0.f;
   for (int t0 = 0; t0 < nvis; t0 += kKeyTile) {
     const int nt = min(kKeyTile, nvis - t0);
     for (int n = slot; n < nt; n += 32) {
       const int nn = t0 + n;
       const int j = nn < nA ? nn : lo + (nn - nA);
       const T* kp = cache + static_cast<long>(bt[j / bs]) * block_stride + koff + (static_cast<long>(g) * bs + j % bs) * dk;
-      float sc = 0.f;
+      float sc[RM];
+#pragma unroll
+      for (int r = 0; r < RM; ++r) sc[r] = 0.f;
 #pragma unroll
       for (int c = 0; c < NC; ++c) {
         const int d = (c * 8 + part) * EL;
@@ -150,33 +161,61 @@ __global__ void __launch_bounds__(256) window_attention_rows_kernel(
           float kf[EL];
           load16(kp + d, kf);
 #pragma unroll
-          for (int e = 0; e < EL; ++e) sc += qf[c][e] * kf[e];
+          for (int r = 0; r < RM; ++r)
+#pragma unroll
+            for (int e = 0; e < EL; ++e) sc[r] += qf[r][c][e] * kf[e];
         }
       }
-      sc += __shfl_xor(sc, 1, 64);
-      sc += __shfl_xor(sc, 2, 64);
-      sc += __shfl_xor(sc, 4, 64);
-      if (part == 0) p[n] = sc;
+#pragma unroll
+      for (int r = 0; r < RM; ++r) {
+        float v = sc[r];
+        v += __shfl_xor(v, 1, 64);
+        v += __shfl_xor(v, 2, 64);
+        v += __shfl_xor(v, 4, 64);
+        if (part == 0) p[r * kKeyTile + n] = v;
+      }
     }
     __syncthreads();
-    const float sc = tid < nt ? p[tid] : -INFINITY;
-    const float m_new = fmaxf(m, block_max(sc, scratch));
-    const float e = tid < nt ? expf(sc - m_new) : 0.f;
-    __syncthreads();  // every score is read before it is replaced by its weight
-    p[tid] = e;
-    const float tsum = block_sum(e, scratch);  // its barriers also publish p
-    const float corr = expf(m - m_new);
-    l = l * corr + tsum;
-    m = m_new;
+    float sv[RM], ev[RM], m_new[RM];
 #pragma unroll
-    for (int c = 0; c < NC; ++c)
+    for (int r = 0; r < RM; ++r) {
+      sv[r] = tid < nt ? p[r * kKeyTile + tid] : -INFINITY;
+      const float wm = wave_max(sv[r]);
+      if (lane == 0) scratch[r * 4 + wid] = wm;
+    }
+    __syncthreads();
 #pragma unroll
-      for (int e2 = 0; e2 < EL; ++e2) acc[c][e2] *= corr;
+    for (int r = 0; r < RM; ++r) {
+      const float mx = fmaxf(fmaxf(scratch[r * 4], scratch[r * 4 + 1]), fmaxf(scratch[r * 4 + 2], scratch[r * 4 + 3]));
+      m_new[r] = fmaxf(m[r], mx);
+      ev[r] = tid < nt ? expf(sv[r] - m_new[r]) : 0.f;
+    }
+    __syncthreads();  // every score and maximum is read before it is replaced
+#pragma unroll
+    for (int r = 0; r < RM; ++r) {
+      p[r * kKeyTile + tid] = ev[r];
+      const float ws = wave_sum(ev[r]);
+      if (lane == 0) scratch[r * 4 + wid] = ws;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < RM; ++r) {
+      const float tsum = (scratch[r * 4] + scratch[r * 4 + 1]) + (scratch[r * 4 + 2] + scratch[r * 4 + 3]);
+      const float corr = expf(m[r] - m_new[r]);  // first tile: exp(-inf) = 0, acc and l are 0
+      l[r] = l[r] * corr + tsum;
+      m[r] = m_new[r];
+#pragma unroll
+      for (int c = 0; c < NC; ++c)
+#pragma unroll
+        for (int e2 = 0; e2 < EL; ++e2) acc[r][c][e2] *= corr;
+    }
     for (int n = slot; n < nt; n += 32) {
       const int nn = t0 + n;
       const int j = nn < nA ? nn : lo + (nn - nA);
       const T* vp = cache + static_cast<long>(bt[j / bs]) * block_stride + voff + (static_cast<long>(g) * bs + j % bs) * dv;
-      const float pn = p[n];
+      float pn[RM];
+#pragma unroll
+      for (int r = 0; r < RM; ++r) pn[r] = p[r * kKeyTile + n];
 #pragma unroll
       for (int c = 0; c < NC; ++c) {
         const int d = (c * 8 + part) * EL;
@@ -184,30 +223,36 @@ __global__ void __launch_bounds__(256) window_attention_rows_kernel(
           float vf[EL];
           load16(vp + d, vf);
 #pragma unroll
-          for (int e2 = 0; e2 < EL; ++e2) acc[c][e2] += pn * vf[e2];
+          for (int r = 0; r < RM; ++r)
+#pragma unroll
+            for (int e2 = 0; e2 < EL; ++e2) acc[r][c][e2] += pn[r] * vf[e2];
         }
       }
     }
-    __syncthreads();  // p is rewritten by the next tile
+    __syncthreads();  // p and scratch are rewritten by the next tile
   }
   // the 8 key slots of a wave that share `part`, then the 4 waves
 #pragma unroll
-  for (int c = 0; c < NC; ++c) {
+  for (int r = 0; r < RM; ++r) {
 #pragma unroll
-    for (int e2 = 0; e2 < EL; ++e2) {
-      float v = acc[c][e2];
-      v += __shfl_xor(v, 8, 64);
-      v += __shfl_xor(v, 16, 64);
-      v += __shfl_xor(v, 32, 64);
-      const int d = (c * 8 + part) * EL + e2;
-      if (lane < 8 && d < dv) red[wid * dv + d] = v;
+    for (int c = 0; c < NC; ++c) {
+#pragma unroll
+      for (int e2 = 0; e2 < EL; ++e2) {
+        float v = acc[r][c][e2];
+        v += __shfl_xor(v, 8, 64);
+        v += __shfl_xor(v, 16, 64);
+        v += __shfl_xor(v, 32, 64);
+        const int d = (c * 8 + part) * EL + e2;
+        if (lane < 8 && d < dv) red[(wid * RM + r) * dv + d] = v;
+      }
     }
+    if (tid == 0) scratch[r] = 1.f / l[r];
   }
   __syncthreads();
-  const float inv = 1.f / l;
-  for (int e2 = tid; e2 < dv; e2 += blockDim.x) {
-    const float o = red[e2] + red[dv + e2] + red[2 * dv + e2] + red[3 * dv + e2];
-    stf(out + static_cast<long>(t) * (H * dv) + hd * dv + e2, o * inv);
+  for (int idx = tid; idx < nr * dv; idx += blockDim.x) {
+    const int r = idx / dv, e2 = idx - r * dv;
+    const float o = (red[r * dv + e2] + red[(RM + r) * dv + e2]) + (red[(2 * RM + r) * dv + e2] + red[(3 * RM + r) * dv + e2]);
+    stf(out + static_cast<long>(t) * (H * dv) + (h0 + r) * dv + e2, o * scratch[r]);
   }
 }
 
@@ -355,14 +400,27 @@ bool launch_window_attention(void* out, const void* q, long q_stride, const void
   const size_t shm = (((dk + 3) & ~3) + kKeyTile + 4 * dv) * sizeof(float);
   if (shm > 60 * 1024) return false;
   if (vec && dv % el == 0 && voff % el == 0 && dk <= 256 && dv <= 256) {  // rows of whole 16-byte pieces
-    if (bf)
-      hipLaunchKernelGGL((window_attention_rows_kernel<bf16_t, 4>), dim3(rows, H), dim3(256), shm, st, (bf16_t*)out,
-                         (const bf16_t*)q, q_stride, (const bf16_t*)cache, block_stride, block_tables, bt_stride, qsl,
-                         seq_lens, S, koff, voff, H, G, dk, dv, bs, scale, window, keep);
-    else
-      hipLaunchKernelGGL((window_attention_rows_kernel<float, 8>), dim3(rows, H), dim3(256), shm, st, (float*)out,
-                         (const float*)q, q_stride, (const float*)cache, block_stride, block_tables, bt_stride, qsl,
-                         seq_lens, S, koff, voff, H, G, dk, dv, bs, scale, window, keep);
+    const int stretch = 8 * el, need = (std::max(dk, dv) + stretch - 1) / stretch;  // 128-byte stretches of a row
+    const int R = H / G;
+#define MIX_ROWS(TT, NC, RM)                                                                                          \
+  do {                                                                                                                \
+    const int nsplit = (R + RM - 1) / RM;                                                                             \
+    const size_t sh = (static_cast<size_t>(RM) * kKeyTile + 4 * RM * dv) * sizeof(float);                             \
+    hipLaunchKernelGGL((window_attention_rows_kernel<TT, NC, RM>), dim3(rows, G * nsplit), dim3(256), sh, st, (TT*)out, \
+                       (const TT*)q, q_stride, (const TT*)cache, block_stride, block_tables, bt_stride, qsl, seq_lens, \
+                       S, koff, voff, H, G, dk, dv, bs, scale, window, keep, nsplit);                                  \
+  } while (0)
+#define MIX_ROWS_T(TT)                                          \
+  do {                                                          \
+    if (need <= 1) { if (R > 1) MIX_ROWS(TT, 1, 8); else MIX_ROWS(TT, 1, 1); } \
+    else if (need <= 2) { if (R > 1) MIX_ROWS(TT, 2, 4); else MIX_ROWS(TT, 2, 1); } \
+    else if (need <= 4) { if (R > 1) MIX_ROWS(TT, 4, 2); else MIX_ROWS(TT, 4, 1); } \
+    else MIX_ROWS(TT, 8, 1);                                    \
+  } while (0)
+    if (bf) MIX_ROWS_T(bf16_t);
+    else MIX_ROWS_T(float);
+#undef MIX_ROWS_T
+#undef MIX_ROWS
     MXS_CHECK_LAUNCH();
     return true;
   }

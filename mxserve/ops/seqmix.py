@@ -204,7 +204,7 @@ def window_attention(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.T
 
 
 # ----------------------------------------------------------------------------- recurrences
-SCAN_PIECE = 256  # tokens per piece of a time-split scan
+SCAN_PIECE = int(os.environ.get("MXS_SCAN_PIECE", "256"))  # tokens per piece of a time-split scan
 SCAN_SCRATCH_BYTES = 512 << 20
 
 
