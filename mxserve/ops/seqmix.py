@@ -204,15 +204,26 @@ def window_attention(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.T
 
 
 # ----------------------------------------------------------------------------- recurrences
-SCAN_PIECE = int(os.environ.get("MXS_SCAN_PIECE", "256"))  # tokens per piece of a time-split scan
+SCAN_PIECE = int(os.environ.get("MXS_SCAN_PIECE", "0"))  # tokens per piece of a time-split scan; 0: by the launch's size
 SCAN_SCRATCH_BYTES = 512 << 20
+SCAN_TARGET_BLOCKS = 1024  # workgroups that fill the 256 CUs four deep
 
 
-def _scan_split(S: int, max_query_len: int, floats: int, device) -> tuple:
+def _scan_split(S: int, T: int, max_query_len: int, floats: int, heads: int, dv: int, device) -> tuple:
     """(piece, npieces, scratch pool, scratch pool) of a scan launch: chunks of 2 pieces or more are cut
-    into pieces that run side by side (two passes and a chaining step, csrc/mixers/scan.hip); the
-    pieces grow until both scratch pools [S, npieces, state] fit SCAN_SCRATCH_BYTES."""
+    into pieces that run side by side (two passes and a chaining step, csrc/mixers/scan.hip).  Pieces
+    are 64 to 256 tokens, as short as it takes to reach SCAN_TARGET_BLOCKS workgroups over the long
+    chunks of the step, and grow until both scratch pools [S, npieces, state] fit SCAN_SCRATCH_BYTES."""
+    max_query_len = min(max_query_len, T)
+    if max_query_len < 128:
+        return 1, 1, None, None
     piece = SCAN_PIECE
+    if piece <= 0:
+        per_piece = heads * -(-dv // 64) * max(1, T // max_query_len)  # workgroups one piece index adds
+        want = -(-SCAN_TARGET_BLOCKS // per_piece)
+        piece = 256
+        while piece > 64 and -(-max_query_len // piece) < want:
+            piece //= 2
     while max_query_len >= 2 * piece:
         n = -(-max_query_len // piece)
         if 2 * S * n * floats * 4 <= SCAN_SCRATCH_BYTES:
@@ -232,7 +243,7 @@ def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.T
     T = q.shape[0]
     if _gpu(q):
         out = torch.empty(T, num_heads * dv, dtype=torch.float32, device=q.device)
-        plan = _scan_split(seq_lens.numel(), min(max_query_len, T), num_heads * dk * dv, q.device)
+        plan = _scan_split(seq_lens.numel(), T, max_query_len, num_heads * dk * dv, num_heads, dv, q.device)
         ext().decay_scan(out, q, k, v, decay, state, state_rows, int(off), qsl, seq_lens, num_heads, dk, dv,
                          bool(silu), *plan)
         return out
@@ -271,8 +282,8 @@ def mlstm_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gates: torch.T
     T = q.shape[0]
     if _gpu(q):
         out = torch.empty(T, num_heads * dv, dtype=torch.float32, device=q.device)
-        plan = _scan_split(seq_lens.numel(), min(max_query_len, T), mlstm_state_floats(num_heads, dk, dv) + num_heads,
-                           q.device)
+        plan = _scan_split(seq_lens.numel(), T, max_query_len, mlstm_state_floats(num_heads, dk, dv) + num_heads,
+                           num_heads, dv, q.device)
         ext().mlstm_scan(out, q, k, v, gates, state, state_rows, int(off), qsl, seq_lens, num_heads, dk, dv,
                          float(gate_cap), float(q_scale), *plan)
         return out
