@@ -108,6 +108,7 @@ def parse(argv=None):
     ap.add_argument("--mixer-prompt", type=int, default=4096)
     ap.add_argument("--mixer-batch", type=int, default=64)
     ap.add_argument("--mixer-context", type=int, default=2048)
+    ap.add_argument("--mixer-only", choices=["all", "voletar", "llama", "kernels"], default="all")
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--iters-per-step", type=int, default=int(os.environ.get("MXS_BENCH_ITERS_PER_STEP", "50")),
@@ -1019,7 +1020,8 @@ def main():
     a = parse()
     if a.mixer_bench:
         from mxserve.tools.mixer_bench import main as mixer_main
-        return mixer_main([int(x) for x in a.mixer_sizes.split(",")], a.mixer_prompt, a.mixer_batch, a.mixer_context)
+        return mixer_main([int(x) for x in a.mixer_sizes.split(",")], a.mixer_prompt, a.mixer_batch, a.mixer_context,
+                          only=a.mixer_only)
     world_env = os.environ.get("WORLD_SIZE")
     if world_env is None and a.gpus > 1:
         return launch_ranks(a)

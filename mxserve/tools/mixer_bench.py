@@ -160,13 +160,16 @@ def kernel_rooflines(width: int, prompt: int, batch: int, context: int) -> list:
     return out
 
 
-def main(sizes: list, prompt: int, batch: int, context: int, layers: int = 4) -> int:
+def main(sizes: list, prompt: int, batch: int, context: int, layers: int = 4, only: str = "all") -> int:
+    """only: all | voletar | llama | kernels (e.g. one model alone under a profiler)."""
     from .. import ops
     ops.ext()
     for width in sizes:
         v, l = register(width, layers)
-        for name in (v, l):
-            print(json.dumps(run_model(name, prompt, batch, context)), flush=True)
-        for e in kernel_rooflines(width, prompt, batch, context):
-            print(json.dumps(e), flush=True)
+        for name, key in ((v, "voletar"), (l, "llama")):
+            if only in ("all", key):
+                print(json.dumps(run_model(name, prompt, batch, context)), flush=True)
+        if only in ("all", "kernels"):
+            for e in kernel_rooflines(width, prompt, batch, context):
+                print(json.dumps(e), flush=True)
     return 0

@@ -97,7 +97,9 @@ def test_each_mixer_alone(dev, portions):
 
 @pytest.mark.parametrize("dev", DEVS)
 @pytest.mark.parametrize("size,keep,target,seen", [(8, 0, 33, True), (8, 0, 32, False), (8, 4, 3, True), (8, 4, 4, False),
-                                                   (1000, 0, 1, True), (1, 0, 39, False), (1, 2, 1, True)])
+                                                   (1000, 0, 1, True), (1, 0, 39, False), (1, 2, 1, True),
+                                                   # the window's first key is a page's first token; the one before it is the previous page's last
+                                                   (9, 0, 32, True), (9, 0, 31, False), (1000, 0, 15, True), (1000, 0, 16, True)])
 def test_one_key_stands_out(dev, size, keep, target, seen):
     """One key far back matches the last query so strongly that the output is that key's value when
     the mask lets it through: the window's edge, the kept first tokens and a far key each decide the
@@ -145,6 +147,21 @@ def test_portions_and_decoding(base, dev, dtype, tol):
         steps = [[("a", p, False)] for p in cut(toks["r0"], sizes)]
         steps[-1] = [("a", steps[-1][0][1], True)]
         _check(replay(eng, steps)["a"], want["r0"], tol)
+    assert eng.kv.num_free() == eng.kv.num_blocks
+
+
+@pytest.mark.parametrize("dev,dtype,tol", [("cpu", "float32", 1e-4), pytest.param("cuda", "float32", 1e-4, marks=pytest.mark.gpu),
+                                           pytest.param("cuda", "bfloat16", 0.12, marks=pytest.mark.gpu)])
+def test_long_decoding(base, dev, dtype, tol):
+    """A short prompt, then well over a hundred tokens one by one: the windows slide off the prompt and
+    over decoded tokens, pages fill and new ones start, the recurrent state is carried all the way."""
+    _skip(dev)
+    path, _, toks, want = base
+    eng = engine(path, dev, dtype, max_tokens=192, eager=(dev == "cpu"))
+    steps = [[("a", p, False)] for p in cut(toks["r4"], [10, 1])]
+    steps[-1] = [("a", steps[-1][0][1], True)]
+    got = replay(eng, steps)["a"]
+    _check(got[8:], want["r4"][8:], tol)
     assert eng.kv.num_free() == eng.kv.num_blocks
 
 
