@@ -260,6 +260,9 @@ class Scheduler:
         for req, n, offsets in plan:
             if n <= 0 or req.num_computed_tokens + n > req.num_known_tokens:
                 raise ValueError(f"{req.request_id}: {n} new tokens do not fit its {req.num_known_tokens} known ones")
+            if req.num_computed_tokens + n > self.max_model_len:  # the runner's block-table rows end there
+                raise ValueError(f"{req.request_id}: {req.num_computed_tokens + n} tokens exceed max_model_len "
+                                 f"{self.max_model_len}")
             if not self.kv.allocate_slots(req, n):
                 raise RuntimeError(f"KV pool exhausted: {req.request_id} needs blocks for {n} more tokens "
                                    f"({self.kv.num_free()} blocks free)")
