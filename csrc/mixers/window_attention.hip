@@ -257,7 +257,7 @@ __global__ void __launch_bounds__(256) window_attention_rows_kernel(
 }
 
 // ---- MFMA form for prompt chunks (bf16, 16-token cache blocks, head sizes multiples of 16 up to
-// 16 * KSM / 16 * VTM).  A wave owns 32 consecutive query rows (two tiles of 16) of one head and walks the visible
+// 16 * KSM / 16 * VTM).  A wave owns 16 consecutive query rows of one head and walks the visible
 // cache blocks (the kept first blocks, then the window's); no LDS, no barriers.  Per block, with
 // v_mfma_f32_16x16x16_bf16:
 //   S^T = K Q^T      A = the block's 16 key rows (8-byte loads from the token-major cache),
@@ -271,8 +271,6 @@ __global__ void __launch_bounds__(256) window_attention_rows_kernel(
 typedef short s4_t __attribute__((ext_vector_type(4)));
 typedef float f4_t __attribute__((ext_vector_type(4)));
 
-constexpr int kQT = 2;  // 16-row query tiles per wave: a key block's K and V operands are loaded once for both
-
 template <int KSM, int VTM>
 __global__ void __launch_bounds__(256) window_attention_mfma_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ cache,
@@ -282,79 +280,67 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(
   const int s = blockIdx.z, hd = blockIdx.y;
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   const int row0 = qsl[s], qlen = qsl[s + 1] - row0;
-  const int qt0 = (blockIdx.x * 4 + wid) * (16 * kQT);  // this wave's first query row inside the chunk
-  if (qt0 >= qlen) return;                              // wave-uniform
-  const int nq = min(16 * kQT, qlen - qt0);
-  const int pos0 = min(max(seq_lens[s] - qlen + qt0, 0), bt_stride * 16 - 16 * kQT);
+  const int qt0 = blockIdx.x * 64 + wid * 16;  // this wave's first query row inside the chunk
+  if (qt0 >= qlen) return;                     // wave-uniform
+  const int nq = min(16, qlen - qt0);
+  const int pos0 = min(max(seq_lens[s] - qlen + qt0, 0), bt_stride * 16 - 16);
   const int g = hd / (H / G);
   const int c = lane & 15, kg = lane >> 4;  // the lane's query (column) and its group of 4 keys / dims
   const int KS = dk >> 4, VT = dv >> 4;
+  const bool qok = c < nq;
+  const int pq = pos0 + c;
   const int* bt = block_tables + static_cast<long>(s) * bt_stride;
-  bool qok[kQT];
-  int pq[kQT];
-  s4_t qf[kQT][KSM];
-#pragma unroll
-  for (int u = 0; u < kQT; ++u) {
-    qok[u] = 16 * u + c < nq;
-    pq[u] = pos0 + 16 * u + c;
-    const bf16_t* qp = q + static_cast<long>(row0 + qt0 + (qok[u] ? 16 * u + c : 0)) * q_stride + hd * dk + 4 * kg;
+  s4_t qf[KSM];
+  {
+    const bf16_t* qp = q + static_cast<long>(row0 + qt0 + (qok ? c : 0)) * q_stride + hd * dk + 4 * kg;
 #pragma unroll
     for (int ks = 0; ks < KSM; ++ks)
-      qf[u][ks] = (ks < KS && qok[u]) ? *reinterpret_cast<const s4_t*>(qp + 16 * ks) : s4_t{0, 0, 0, 0};
+      qf[ks] = (ks < KS && qok) ? *reinterpret_cast<const s4_t*>(qp + 16 * ks) : s4_t{0, 0, 0, 0};
   }
   const int p_last = pos0 + nq - 1;
   const int lo_first = window > 0 ? max(pos0 - window + 1, 0) : 0;
   const int wb = lo_first >> 4, lastb = p_last >> 4;
   const int kA = window > 0 ? min((keep + 15) >> 4, wb) : 0;  // kept first blocks below the window's
-  float m[kQT], l[kQT];
-  f4_t o[kQT][VTM];
+  float m = -INFINITY, l = 0.f;
+  f4_t o[VTM];
 #pragma unroll
-  for (int u = 0; u < kQT; ++u) {
-    m[u] = -INFINITY;
-    l[u] = 0.f;
-#pragma unroll
-    for (int vt = 0; vt < VTM; ++vt) o[u][vt] = f4_t{0.f, 0.f, 0.f, 0.f};
-  }
+  for (int vt = 0; vt < VTM; ++vt) o[vt] = f4_t{0.f, 0.f, 0.f, 0.f};
   const int nit = kA + (lastb - wb + 1);
   for (int it = 0; it < nit; ++it) {
     const int kb = it < kA ? it : wb + (it - kA);
     const bf16_t* blk = cache + static_cast<long>(bt[kb]) * block_stride;
+    f4_t acc = f4_t{0.f, 0.f, 0.f, 0.f};
     const bf16_t* kp = blk + koff + (static_cast<long>(g) * 16 + c) * dk + 4 * kg;
-    s4_t ak[KSM];
 #pragma unroll
     for (int ks = 0; ks < KSM; ++ks)
-      if (ks < KS) ak[ks] = *reinterpret_cast<const s4_t*>(kp + 16 * ks);
-    s4_t ph[kQT], pl[kQT];
-    float corr[kQT];
+      if (ks < KS)
+        acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(*reinterpret_cast<const s4_t*>(kp + 16 * ks), qf[ks], acc, 0, 0, 0);
+    float sv[4], mx = -INFINITY;
 #pragma unroll
-    for (int u = 0; u < kQT; ++u) {
-      f4_t acc = f4_t{0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < 4; ++i) {
+      const int j = kb * 16 + 4 * kg + i;
+      const bool vis = qok && j <= pq && (window <= 0 || pq - j < window || j < keep);
+      sv[i] = vis ? acc[i] * scale : -INFINITY;
+      mx = fmaxf(mx, sv[i]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float corr = m_new == -INFINITY ? 1.f : expf(m - m_new);
+    float pr[4], ps = 0.f;
 #pragma unroll
-      for (int ks = 0; ks < KSM; ++ks)
-        if (ks < KS) acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ak[ks], qf[u][ks], acc, 0, 0, 0);
-      float sv[4], mx = -INFINITY;
+    for (int i = 0; i < 4; ++i) {
+      pr[i] = sv[i] == -INFINITY ? 0.f : expf(sv[i] - m_new);
+      ps += pr[i];
+    }
+    l = l * corr + ps;
+    m = m_new;
+    s4_t ph, pl;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int j = kb * 16 + 4 * kg + i;
-        const bool vis = qok[u] && j <= pq[u] && (window <= 0 || pq[u] - j < window || j < keep);
-        sv[i] = vis ? acc[i] * scale : -INFINITY;
-        mx = fmaxf(mx, sv[i]);
-      }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m[u], mx);
-      corr[u] = m_new == -INFINITY ? 1.f : expf(m[u] - m_new);
-      float ps = 0.f;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float pr = sv[i] == -INFINITY ? 0.f : expf(sv[i] - m_new);
-        ps += pr;
-        const bf16_t hi = f2bf(pr);
-        ph[u][i] = static_cast<short>(hi);
-        pl[u][i] = static_cast<short>(f2bf(pr - bf2f(hi)));
-      }
-      l[u] = l[u] * corr[u] + ps;
-      m[u] = m_new;
+    for (int i = 0; i < 4; ++i) {
+      const bf16_t hi = f2bf(pr[i]);
+      ph[i] = static_cast<short>(hi);
+      pl[i] = static_cast<short>(f2bf(pr[i] - bf2f(hi)));
     }
     const bf16_t* vp = blk + voff + (static_cast<long>(g) * 16 + 4 * kg) * dv + c;
 #pragma unroll
@@ -364,34 +350,26 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(
 #pragma unroll
         for (int j = 0; j < 4; ++j)  // rows past the sequence's last token may hold anything: read them as 0
           a[j] = (kb * 16 + 4 * kg + j <= p_last) ? static_cast<short>(vp[static_cast<long>(j) * dv + 16 * vt]) : short(0);
+        f4_t t = o[vt];
 #pragma unroll
-        for (int u = 0; u < kQT; ++u) {
-          f4_t t = o[u][vt];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) t[i] *= corr[u];
-          t = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, ph[u], t, 0, 0, 0);
-          o[u][vt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pl[u], t, 0, 0, 0);
-        }
+        for (int i = 0; i < 4; ++i) t[i] *= corr;
+        t = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, ph, t, 0, 0, 0);
+        o[vt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pl, t, 0, 0, 0);
       }
     }
   }
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (!qok) return;
+  const float inv = 1.f / l;
+  bf16_t* op = out + static_cast<long>(row0 + qt0 + c) * (H * dv) + hd * dv + 4 * kg;
 #pragma unroll
-  for (int u = 0; u < kQT; ++u) {
-    float lt = l[u];
-    lt += __shfl_xor(lt, 16, 64);
-    lt += __shfl_xor(lt, 32, 64);
-    if (qok[u]) {
-      const float inv = 1.f / lt;
-      bf16_t* op = out + static_cast<long>(row0 + qt0 + 16 * u + c) * (H * dv) + hd * dv + 4 * kg;
-#pragma unroll
-      for (int vt = 0; vt < VTM; ++vt) {
-        if (vt < VT) {
-          uint2 w;
-          w.x = pack2(o[u][vt][0] * inv, o[u][vt][1] * inv);
-          w.y = pack2(o[u][vt][2] * inv, o[u][vt][3] * inv);
-          *reinterpret_cast<uint2*>(op + 16 * vt) = w;
-        }
-      }
+  for (int vt = 0; vt < VTM; ++vt) {
+    if (vt < VT) {
+      uint2 w;
+      w.x = pack2(o[vt][0] * inv, o[vt][1] * inv);
+      w.y = pack2(o[vt][2] * inv, o[vt][3] * inv);
+      *reinterpret_cast<uint2*>(op + 16 * vt) = w;
     }
   }
 }
@@ -405,7 +383,7 @@ bool launch_window_attention(void* out, const void* q, long q_stride, const void
   // tokens ride along as 1-row tiles); everything else the scalar form below
   if (bf && max_q >= 16 && bs == 16 && dk % 16 == 0 && dv % 16 == 0 && dk <= 128 && dv <= 128 && q_stride % 4 == 0 &&
       reinterpret_cast<uintptr_t>(q) % 8 == 0 && koff % 4 == 0 && voff % 4 == 0 && block_stride % 4 == 0) {
-    const dim3 grid((max_q + 64 * kQT - 1) / (64 * kQT), H, S);
+    const dim3 grid((max_q + 63) / 64, H, S);
 #define MIX_WA(KSM, VTM)                                                                                              \
   hipLaunchKernelGGL((window_attention_mfma_kernel<KSM, VTM>), grid, dim3(256), 0, st, (bf16_t*)out, (const bf16_t*)q, \
                      q_stride, (const bf16_t*)cache, block_stride, block_tables, bt_stride, qsl, seq_lens, koff, voff, \
