@@ -645,7 +645,8 @@ class ModelRunner:
         if not buckets:
             log.warning("no decode bucket has graph-capturable collectives; decode runs eagerly")
             return
-        if tune and "l0.qkv" in m.w:  # the transformer families' projections
+        # a model without tunable projections (its tunable_shapes() is empty) runs the library's choice
+        if tune and (not hasattr(m, "tunable_shapes") or m.tunable_shapes()):
             self._tune_gemms(buckets)
         self._capture(buckets)
 

@@ -19,7 +19,6 @@ linear attention S [H, dk, dv] at `off`; mLSTM S [H, dk, dv], then n [H, dk], th
 from __future__ import annotations
 
 import importlib
-import math
 import os
 import threading
 from typing import Optional
@@ -314,7 +313,3 @@ def mlstm_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gates: torch.T
             den = torch.maximum((n * qf[t]).sum(-1).abs(), torch.exp(-m)) + 1e-6
             out[t] = torch.einsum("hdv,hd->hv", S, qf[t]) / den.unsqueeze(1)
     return out.reshape(T, H * dv)
-
-
-def sqrt_inv(d: int) -> float:
-    return 1.0 / math.sqrt(d)

@@ -269,3 +269,32 @@ def test_greedy_generation_through_the_scheduler(base, dev, dtype):
         for row, tok in zip(lg, o):
             assert row[tok] >= row.max() - margin * (row.max() - row.min())
     assert eng.kv.num_free() == eng.kv.num_blocks
+
+
+def test_trace_runner_command_line(base, tmp_path):
+    """bin/trace_run as a user starts it: steps on stdin, `done <step>` after each, logits files for the
+    steps that want some, pages and slots given back under --max-tokens."""
+    import json
+    import os
+    import subprocess
+    import sys
+    path, _, toks, want = base
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    t = toks["r1"]
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": t[:20], "want": [0, 19]}], "end": []},
+             {"step": 1, "entries": [{"id": "x", "tokens": t[20:22], "want": []}, {"id": "y", "tokens": toks["r2"], "want": [0]}],
+              "end": ["y"]},
+             {"step": 2, "entries": [{"id": "x", "tokens": t[22:], "want": [len(t) - 23]}], "end": ["x"]}]
+    out = tmp_path / "out"
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(path), "--dtype", "float32",
+                        "--out", str(out), "--max-tokens", "128", "--device", "cpu"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    V = BASE["vocab"]
+    a = np.fromfile(out / "0.f32", dtype="<f4").reshape(-1, V)
+    b = np.fromfile(out / "1.f32", dtype="<f4").reshape(-1, V)
+    c = np.fromfile(out / "2.f32", dtype="<f4").reshape(-1, V)
+    _check(a.astype(np.float64), want["r1"][[0, 19]], 1e-4)
+    _check(b.astype(np.float64), want["r2"][[0]], 1e-4)
+    _check(c.astype(np.float64), want["r1"][[len(t) - 1]], 1e-4)
