@@ -307,34 +307,15 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(
   for (int vt = 0; vt < VTM; ++vt) o[vt] = f4_t{0.f, 0.f, 0.f, 0.f};
   const float sl2 = scale * 1.4426950408889634f;
   const int nit = kA + (lastb - wb + 1);
-  // operands of a key block: K rows (A of S^T) and gathered V^T (A of O^T); the next block's are
-  // loaded while this block's are used (the loop is bound by load latency, not by arithmetic)
-  s4_t ak0[KSM], av0[VTM], ak1[KSM], av1[VTM];
-  auto load_block = [&](int it, s4_t* k_out, s4_t* v_out) {
+  for (int it = 0; it < nit; ++it) {
     const int kb = it < kA ? it : wb + (it - kA);
     const bf16_t* blk = cache + static_cast<long>(bt[kb]) * block_stride;
+    f4_t acc = f4_t{0.f, 0.f, 0.f, 0.f};
     const bf16_t* kp = blk + koff + (static_cast<long>(g) * 16 + c) * dk + 4 * kg;
 #pragma unroll
     for (int ks = 0; ks < KSM; ++ks)
-      if (ks < KS) k_out[ks] = *reinterpret_cast<const s4_t*>(kp + 16 * ks);
-    const bf16_t* vp = blk + voff + (static_cast<long>(g) * 16 + 4 * kg) * dv + c;
-    const int k0 = kb * 16;
-    const bool vall = k0 + 15 <= p_last;
-#pragma unroll
-    for (int vt = 0; vt < VTM; ++vt) {
-      if (vt < VT) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)  // rows past the sequence's last token may hold anything: read them as 0
-          v_out[vt][j] = (vall || k0 + 4 * kg + j <= p_last) ? static_cast<short>(vp[static_cast<long>(j) * dv + 16 * vt]) : short(0);
-      }
-    }
-  };
-  auto use_block = [&](int it, const s4_t* ak, const s4_t* av) {
-    const int kb = it < kA ? it : wb + (it - kA);
-    f4_t acc = f4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int ks = 0; ks < KSM; ++ks)
-      if (ks < KS) acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ak[ks], qf[ks], acc, 0, 0, 0);
+      if (ks < KS)
+        acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(*reinterpret_cast<const s4_t*>(kp + 16 * ks), qf[ks], acc, 0, 0, 0);
     // a block that every query of the tile sees whole (the usual case inside a window) needs no mask
     const int k0 = kb * 16;
     const bool whole = k0 + 15 <= pos0 && (window <= 0 || k0 >= p_last - window + 1 || k0 + 15 < keep);
@@ -376,21 +357,18 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(
       ph[i] = static_cast<short>(uh >> 16);
       pl[i] = static_cast<short>(ul >> 16);
     }
+    const bf16_t* vp = blk + voff + (static_cast<long>(g) * 16 + 4 * kg) * dv + c;
+    const bool vall = k0 + 15 <= p_last;
 #pragma unroll
     for (int vt = 0; vt < VTM; ++vt) {
       if (vt < VT) {
-        f4_t t = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(av[vt], ph, o[vt], 0, 0, 0);
-        o[vt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(av[vt], pl, t, 0, 0, 0);
+        s4_t a;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)  // rows past the sequence's last token may hold anything: read them as 0
+          a[j] = (vall || k0 + 4 * kg + j <= p_last) ? static_cast<short>(vp[static_cast<long>(j) * dv + 16 * vt]) : short(0);
+        f4_t t = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, ph, o[vt], 0, 0, 0);
+        o[vt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pl, t, 0, 0, 0);
       }
-    }
-  };
-  load_block(0, ak0, av0);
-  for (int it = 0; it < nit; it += 2) {  // two blocks per trip, so that each buffer keeps its registers
-    if (it + 1 < nit) load_block(it + 1, ak1, av1);
-    use_block(it, ak0, av0);
-    if (it + 1 < nit) {
-      if (it + 2 < nit) load_block(it + 2, ak0, av0);
-      use_block(it + 1, ak1, av1);
     }
   }
   l += __shfl_xor(l, 16, 64);
