@@ -258,7 +258,7 @@ __global__ void __launch_bounds__(256) window_attention_rows_kernel(
 
 // ---- MFMA form for prompt chunks (bf16, 16-token cache blocks, head sizes multiples of 16 up to
 // 16 * KSM / 16 * VTM).  A wave owns 16 consecutive query rows of one head and walks the visible
-// cache blocks (the kept first blocks, then the window's); no LDS, no barriers.  Per block, with
+// cache blocks (the kept first blocks, then the window's); no workgroup barriers.  Per block, with
 // v_mfma_f32_16x16x16_bf16:
 //   S^T = K Q^T      A = the block's 16 key rows (8-byte loads from the token-major cache),
 //                    B = Q^T, held in registers for the whole walk.  The accumulator has the query
@@ -266,7 +266,8 @@ __global__ void __launch_bounds__(256) window_attention_rows_kernel(
 //                    work plus two cross-lane exchanges.
 //   O^T += V^T P^T   B = P^T straight from the S^T accumulator's registers; every weight is split
 //                    into two bf16 halves (p = hi + lo, two MFMAs) so the product keeps 16 mantissa
-//                    bits of the fp32 weight; A = V^T gathered from the token-major value rows.
+//                    bits of the fp32 weight; A = V^T: the block's token-major value rows go through
+//                    the wave's LDS area (16-byte pieces in, 2-byte reads out, key-contiguous).
 // Scores, maxima, sums and the output accumulator are fp32.
 typedef short s4_t __attribute__((ext_vector_type(4)));
 typedef float f4_t __attribute__((ext_vector_type(4)));
@@ -277,11 +278,17 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(
     long block_stride, const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ qsl,
     const int* __restrict__ seq_lens, int koff, int voff, int H, int G, int dk, int dv, float scale, int window,
     int keep) {
+  // each wave's own staging area for a block's value rows (token-major in the pages): written with
+  // 16-byte pieces, read back as the key-contiguous V^T operand.  Rows are padded by 8 elements so
+  // that the four key groups of a read fall into different banks.
+  __shared__ __attribute__((aligned(16))) bf16_t vlds[4][16 * (16 * VTM + 8)];
   const int s = blockIdx.z, hd = blockIdx.y;
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  bf16_t* vw = vlds[wid];
+  const int DVP = dv + 8;
   const int row0 = qsl[s], qlen = qsl[s + 1] - row0;
   const int qt0 = blockIdx.x * 64 + wid * 16;  // this wave's first query row inside the chunk
-  if (qt0 >= qlen) return;                     // wave-uniform
+  if (qt0 >= qlen) return;                     // wave-uniform (no workgroup barrier is used below)
   const int nq = min(16, qlen - qt0);
   const int pos0 = min(max(seq_lens[s] - qlen + qt0, 0), bt_stride * 16 - 16);
   const int g = hd / (H / G);
@@ -342,14 +349,26 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(
       ph[i] = static_cast<short>(hi);
       pl[i] = static_cast<short>(f2bf(pr[i] - bf2f(hi)));
     }
-    const bf16_t* vp = blk + voff + (static_cast<long>(g) * 16 + 4 * kg) * dv + c;
+    // the block's 16 value rows are one contiguous stretch of 16 * dv elements
+    const bf16_t* vblk = blk + voff + static_cast<long>(g) * 16 * dv;
+    __builtin_amdgcn_wave_barrier();  // the previous block's reads come first
+#pragma unroll
+    for (int r = 0; r < (VTM + 1) / 2; ++r) {
+      const int idx = lane + 64 * r;  // 16-byte piece
+      if (idx < 2 * dv) {
+        const int e0 = idx * 8, vr = e0 / dv, vc = e0 - vr * dv;
+        *reinterpret_cast<uint4*>(vw + vr * DVP + vc) = *reinterpret_cast<const uint4*>(vblk + e0);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+    const bf16_t* vp = vw + 4 * kg * DVP + c;
 #pragma unroll
     for (int vt = 0; vt < VTM; ++vt) {
       if (vt < VT) {
         s4_t a;
 #pragma unroll
         for (int j = 0; j < 4; ++j)  // rows past the sequence's last token may hold anything: read them as 0
-          a[j] = (kb * 16 + 4 * kg + j <= p_last) ? static_cast<short>(vp[static_cast<long>(j) * dv + 16 * vt]) : short(0);
+          a[j] = (kb * 16 + 4 * kg + j <= p_last) ? static_cast<short>(vp[j * DVP + 16 * vt]) : short(0);
         f4_t t = o[vt];
 #pragma unroll
         for (int i = 0; i < 4; ++i) t[i] *= corr;
@@ -382,7 +401,7 @@ bool launch_window_attention(void* out, const void* q, long q_stride, const void
   // prompt chunks in bf16 with MFMA-shaped heads: the matrix-core form (rows of a mixed step's single
   // tokens ride along as 1-row tiles); everything else the scalar form below
   if (bf && max_q >= 16 && bs == 16 && dk % 16 == 0 && dv % 16 == 0 && dk <= 128 && dv <= 128 && q_stride % 4 == 0 &&
-      reinterpret_cast<uintptr_t>(q) % 8 == 0 && koff % 4 == 0 && voff % 4 == 0 && block_stride % 4 == 0) {
+      reinterpret_cast<uintptr_t>(q) % 8 == 0 && koff % 8 == 0 && voff % 8 == 0 && block_stride % 8 == 0) {
     const dim3 grid((max_q + 63) / 64, H, S);
 #define MIX_WA(KSM, VTM)                                                                                              \
   hipLaunchKernelGGL((window_attention_mfma_kernel<KSM, VTM>), grid, dim3(256), 0, st, (bf16_t*)out, (const bf16_t*)q, \
