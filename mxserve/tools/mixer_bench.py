@@ -53,6 +53,7 @@ def register(width: int, layers: int) -> tuple:
 
 
 def _time(fn, reps: int) -> float:
+    fn()  # code objects loaded, allocator warm
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(reps):
