@@ -308,10 +308,11 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(
   const int lo_first = window > 0 ? max(pos0 - window + 1, 0) : 0;
   const int wb = lo_first >> 4, lastb = p_last >> 4;
   const int kA = window > 0 ? min((keep + 15) >> 4, wb) : 0;  // kept first blocks below the window's
-  float m = -INFINITY, l = 0.f;
+  float m = -INFINITY, l = 0.f;  // m in log2 units: scores are scaled by scale * log2(e), weights are exp2
   f4_t o[VTM];
 #pragma unroll
   for (int vt = 0; vt < VTM; ++vt) o[vt] = f4_t{0.f, 0.f, 0.f, 0.f};
+  const float sl2 = scale * 1.4426950408889634f;
   const int nit = kA + (lastb - wb + 1);
   for (int it = 0; it < nit; ++it) {
     const int kb = it < kA ? it : wb + (it - kA);
@@ -322,32 +323,46 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(
     for (int ks = 0; ks < KSM; ++ks)
       if (ks < KS)
         acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(*reinterpret_cast<const s4_t*>(kp + 16 * ks), qf[ks], acc, 0, 0, 0);
+    // a block that every query of the tile sees whole (the usual case inside a window) needs no mask
+    const int k0 = kb * 16;
+    const bool whole = k0 + 15 <= pos0 && (window <= 0 || k0 >= p_last - window + 1 || k0 + 15 < keep);
     float sv[4], mx = -INFINITY;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int j = kb * 16 + 4 * kg + i;
-      const bool vis = qok && j <= pq && (window <= 0 || pq - j < window || j < keep);
-      sv[i] = vis ? acc[i] * scale : -INFINITY;
+      if (whole) {
+        sv[i] = acc[i] * sl2;
+      } else {
+        const int j = k0 + 4 * kg + i;
+        const bool vis = qok && j <= pq && (window <= 0 || pq - j < window || j < keep);
+        sv[i] = vis ? acc[i] * sl2 : -INFINITY;
+      }
       mx = fmaxf(mx, sv[i]);
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float m_new = fmaxf(m, mx);
-    const float corr = m_new == -INFINITY ? 1.f : expf(m - m_new);
-    float pr[4], ps = 0.f;
+    // the running maximum seldom moves after the first blocks: rescale only when some query's did
+    if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {
+      const float corr = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
+      l *= corr;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      pr[i] = sv[i] == -INFINITY ? 0.f : expf(sv[i] - m_new);
-      ps += pr[i];
+      for (int vt = 0; vt < VTM; ++vt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[vt][i] *= corr;
+      m = m_new;
     }
-    l = l * corr + ps;
-    m = m_new;
     s4_t ph, pl;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const bf16_t hi = f2bf(pr[i]);
-      ph[i] = static_cast<short>(hi);
-      pl[i] = static_cast<short>(f2bf(pr[i] - bf2f(hi)));
+      // exp2(-inf) = 0; a query with nothing visible yet (m = -inf) must not turn -inf - -inf into a weight
+      const float pr = (whole || sv[i] != -INFINITY) ? __builtin_amdgcn_exp2f(sv[i] - m) : 0.f;
+      l += pr;
+      // pr = hi + lo: hi the upper 16 bits (exact), lo = pr - hi rounded to bf16 (pr >= 0, finite)
+      const uint32_t u = __float_as_uint(pr), uh = u & 0xFFFF0000u;
+      uint32_t ul = __float_as_uint(pr - __uint_as_float(uh));
+      ul += 0x7FFFu + ((ul >> 16) & 1u);
+      ph[i] = static_cast<short>(uh >> 16);
+      pl[i] = static_cast<short>(ul >> 16);
     }
     // the block's 16 value rows are one contiguous stretch of 16 * dv elements
     const bf16_t* vblk = blk + voff + static_cast<long>(g) * 16 * dv;
@@ -362,17 +377,15 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(
     }
     __builtin_amdgcn_wave_barrier();
     const bf16_t* vp = vw + 4 * kg * DVP + c;
+    const bool vall = k0 + 15 <= p_last;
 #pragma unroll
     for (int vt = 0; vt < VTM; ++vt) {
       if (vt < VT) {
         s4_t a;
 #pragma unroll
         for (int j = 0; j < 4; ++j)  // rows past the sequence's last token may hold anything: read them as 0
-          a[j] = (kb * 16 + 4 * kg + j <= p_last) ? static_cast<short>(vp[j * DVP + 16 * vt]) : short(0);
-        f4_t t = o[vt];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) t[i] *= corr;
-        t = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, ph, t, 0, 0, 0);
+          a[j] = (vall || k0 + 4 * kg + j <= p_last) ? static_cast<short>(vp[j * DVP + 16 * vt]) : short(0);
+        const f4_t t = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, ph, o[vt], 0, 0, 0);
         o[vt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pl, t, 0, 0, 0);
       }
     }
