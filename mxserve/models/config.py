@@ -18,7 +18,7 @@ from typing import Optional
 @dataclass
 class ModelConfig:
     name: str
-    arch: str  # "llama" | "qwen3" | "mixtral" | "voletar"
+    arch: str  # "llama" | "qwen3" | "mixtral" | "voletar" | "tapasun"
     hidden_size: int
     intermediate_size: int
     num_layers: int
@@ -40,9 +40,10 @@ class ModelConfig:
     bos_token_id: Optional[int] = None
     eos_token_ids: list = field(default_factory=list)
     chat_template: str = "llama3"
-    # designs whose layers differ from one another (arch "voletar"): the checkpoint's own config.json
-    # structure -- per-layer mixer type and sizes, the looped span, norm eps, logit soft-cap -- as
-    # mxserve/models/voletar.py reads it.  None for the uniform transformer families.
+    # designs whose layers differ from one another (arch "voletar", "tapasun"): the checkpoint's own
+    # config.json structure -- per-layer mixer type and sizes, norm eps and the design's other
+    # constants -- as the design's module (mxserve/models/<arch>.py) reads it.  None for the uniform
+    # transformer families.
     arch_config: Optional[dict] = None
 
     @property
@@ -51,9 +52,10 @@ class ModelConfig:
 
     @property
     def has_recurrent_state(self) -> bool:
-        """Layers that carry a per-sequence state from token to token (linear attention, mLSTM): no
-        prefix caching (a cached block has no state to resume from) and one state slot per request."""
-        return self.arch == "voletar"
+        """Layers that carry a per-sequence state from token to token (linear attention, mLSTM, state
+        spaces, delta rule, short convolutions): no prefix caching (a cached block has no state to
+        resume from) and one state slot per request."""
+        return self.arch in ("voletar", "tapasun")
 
     @property
     def q_size(self) -> int:
@@ -65,14 +67,16 @@ class ModelConfig:
 
     def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
         if self.arch_config is not None:
-            from .voletar import layer_plan
-            return sum(r.kv_heads * (r.dk + r.dv) for r in layer_plan(self.arch_config).attn_runs) * dtype_bytes
+            from .hybrid import design_module
+            plan = design_module(self.arch).layer_plan(self.arch_config)
+            return sum(r.kv_heads * (r.dk + r.dv) for r in plan.attn_runs) * dtype_bytes
         return self.num_layers * 2 * self.num_kv_heads * self.head_dim * dtype_bytes
 
     def num_params(self) -> int:
         if self.arch_config is not None:
-            from .voletar import weight_shapes
-            return sum(int(__import__("math").prod(v)) for v in weight_shapes(self.arch_config).values())
+            from .hybrid import design_module
+            shapes = design_module(self.arch).weight_shapes(self.arch_config)
+            return sum(int(__import__("math").prod(v)) for v in shapes.values())
         h, i, L = self.hidden_size, self.intermediate_size, self.num_layers
         attn = h * (self.q_size + 2 * self.kv_size) + self.q_size * h
         if self.is_moe:
@@ -203,9 +207,50 @@ _reg(voletar_config("tiny-voletar", {
                    "right": {"heads": 4, "dim": 32, "vdim": 16, "gate_cap": 8.0}}}]}))
 
 
+def tapasun_config(name: str, d: dict) -> ModelConfig:
+    """A Tapasun checkpoint's config.json: `width`, `vocab`, `embedding.scale`, `norm.eps`, `layers` (each
+    with `type` mamba2 | attention | parallel, `mixer`, `mlp` or null).  The uniform fields are filled
+    from the first attention for the code that sizes things from them (profiler, planner)."""
+    layers = d["layers"]
+    atts = [l["mixer"].get("left", l["mixer"]) for l in layers if l["type"] in ("attention", "parallel")]
+    att = atts[0] if atts else {"heads": 1, "kv_heads": 1, "dim": int(d["width"])}
+    ffs = [l["mlp"]["ff"] for l in layers if l.get("mlp")]
+    keep = {k: d[k] for k in ("layers", "norm", "embedding", "width", "vocab") if k in d}
+    return ModelConfig(
+        name=name, arch="tapasun", hidden_size=int(d["width"]), intermediate_size=max(ffs) if ffs else 0,
+        num_layers=len(layers), num_heads=int(att["heads"]), num_kv_heads=int(att.get("kv_heads", att["heads"])),
+        head_dim=int(att["dim"]), vocab_size=int(d["vocab"]), rms_norm_eps=float((d.get("norm") or {}).get("eps", 1e-5)),
+        tie_word_embeddings=False, max_position_embeddings=int(d.get("max_position_embeddings", 1 << 20)),
+        bos_token_id=d.get("bos_token_id"), eos_token_ids=list(d.get("eos_token_ids") or []),
+        chat_template="chatml", arch_config=keep)
+
+
+# A small Tapasun (random weights) with every kind of layer, a layer without feed-forward and shared pages.
+_reg(tapasun_config("tiny-tapasun", {
+    "architecture": "Tapasun", "width": 96, "vocab": 384, "norm": {"eps": 1e-5}, "embedding": {"scale": 4.0},
+    "layers": [
+        {"type": "attention", "mlp": {"kind": "dense", "ff": 160},
+         "mixer": {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 16, "scale": 0.2,
+                   "rot": {"dims": 16, "base": 10000.0,
+                           "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 64}}}},
+        {"type": "mamba2", "mlp": None,
+         "mixer": {"heads": 3, "vdim": 16, "state": 24, "groups": 1, "conv": 4, "norm_groups": 3}},
+        {"type": "parallel", "mlp": {"kind": "dense", "ff": 128}, "mixer": {
+            "left": {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 32, "scale": 0.3,
+                     "rot": {"dims": 8, "base": 10000.0, "scaling": {"factor": 2.0}}},
+            "right": {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 24, "conv": 3},
+            "left_scale": 0.7, "right_scale": 1.3}},
+        {"type": "attention", "mlp": {"kind": "dense", "ff": 160},
+         "mixer": {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 16, "scale": 0.2, "kv_from": 0,
+                   "rot": {"dims": 16, "base": 10000.0,
+                           "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 64}}}}]}))
+
+
 def _from_hf_json(name: str, d: dict) -> ModelConfig:
     if d.get("architecture") == "Voletar":
         return voletar_config(name, d)
+    if d.get("architecture") == "Tapasun":
+        return tapasun_config(name, d)
     arch_list = d.get("architectures") or []
     mt = d.get("model_type", "")
     if "qwen3" in mt or any("Qwen3" in a for a in arch_list):

@@ -519,4 +519,7 @@ def build_model(cfg: ModelConfig, device, dtype=torch.bfloat16, moe_dispatch: st
     if cfg.arch == "voletar":
         from .voletar import VoletarLM
         return VoletarLM(cfg, device, dtype, block_size)
+    if cfg.arch == "tapasun":
+        from .tapasun import TapasunLM
+        return TapasunLM(cfg, device, dtype, block_size)
     return TransformerLM(cfg, device, dtype, moe_dispatch)

@@ -11,11 +11,23 @@ in a slot) and computes its output from a step's flattened token batch.
                         per-head unit norm, sigmoid output gate
   ParallelPair          two mixers reading the same input; the layer averages their outputs after
                         an RMSNorm of each over the model width
+  RotaryAttention       softmax attention with interleaved rotary pairs on part of each head (plain,
+                        linearly scaled or band-scaled frequencies), optional per-head q/k RMS norm,
+                        a sink in the softmax denominator (fixed or learned per head), optionally
+                        values turned by their position and outputs turned back, optionally reading
+                        another layer's pages instead of projecting keys and values
+  Mamba2                selective state space with a scalar decay per head and token, short causal
+                        convolution, SiLU gate before a grouped RMS norm
+  GatedDeltaRule        delta-rule matrix memory with a decay per head and key channel, short
+                        convolutions and unit-norm q/k, per-head RMS norm and a sigmoid output gate
+  ScaledPair            two mixers reading the same input, summed with fixed scales through one
+                        output projection over their concatenated activations
 
 The kernels are in mxserve/ops/seqmix.py (csrc/mixers/*.hip on the GPU).
 """
 from __future__ import annotations
 
+import math
 from dataclasses import dataclass
 from typing import Optional
 
@@ -173,6 +185,263 @@ class ParallelPair(Mixer):
         a = self.left.forward(parts[:nl], h, w, ctx, koff, voff, soff)
         b = self.right.forward(parts[nl:], h, w, ctx, koff, voff, soff)
         return a, b
+
+
+def rotary_frequencies(dims: int, base: float, scaling: Optional[dict] = None) -> torch.Tensor:
+    """fp32 [dims / 2]: base^(-2i/dims), computed in float64 on the host.  scaling {factor}: every
+    frequency divided by factor.  scaling {factor, low, high, original}: by wavelength l = 2 pi / f,
+    kept where l < original / high, divided by factor where l > original / low, and in between blended
+    with s = (original / l - low) / (high - low) as (1 - s) f / factor + s f."""
+    f = [float(base) ** (-2.0 * i / dims) for i in range(dims // 2)]
+    if scaling:
+        factor = float(scaling["factor"])
+        if "original" in scaling:
+            orig, low, high = float(scaling["original"]), float(scaling["low"]), float(scaling["high"])
+            out = []
+            for fi in f:
+                wave = 2.0 * math.pi / fi
+                if wave < orig / high:
+                    out.append(fi)
+                elif wave > orig / low:
+                    out.append(fi / factor)
+                else:
+                    sm = (orig / wave - low) / (high - low)
+                    out.append((1.0 - sm) * fi / factor + sm * fi)
+            f = out
+        else:
+            f = [fi / factor for fi in f]
+    return torch.tensor(f, dtype=torch.float64).to(torch.float32)
+
+
+def _fp32(w: dict, name: str) -> None:
+    """Constants of a recurrence, a sink or a decay are read as fp32 by the kernels."""
+    w[name] = w[name].to(torch.float32).contiguous()
+
+
+class RotaryAttention(Mixer):
+    """sink: None (plain softmax) | "zero" (the denominator holds one more exp(0)) | "learned" (tensor
+    `<prefix>sink` [heads]).  rot: {dims, base, scaling}.  rotate_values: the cached value of position j
+    is turned by j over all of vdim (plain frequencies of rot.base) and a head's output at position i
+    is turned back by i.  kv_from: the layer whose pages this mixer reads; it has no k / v tensors."""
+
+    def __init__(self, prefix: str, width: int, heads: int, kv_heads: int, dim: int, vdim: int, scale: float,
+                 rot: dict, qk_norm: bool, sink: Optional[str], rotate_values: bool = False,
+                 kv_from: Optional[int] = None):
+        if heads % kv_heads:
+            raise ValueError(f"{prefix}: {heads} query heads do not divide over {kv_heads} kv heads")
+        rd = int(rot["dims"])
+        if rd % 2 or rd > dim or (rotate_values and vdim % 2):
+            raise ValueError(f"{prefix}: rotary pairs need an even number of dimensions inside the head")
+        if sink not in (None, "zero", "learned"):
+            raise ValueError(f"{prefix}: unknown sink {sink!r}")
+        self.p, self.width = prefix, width
+        self.heads, self.kv_heads, self.dk, self.dv = heads, kv_heads, dim, vdim
+        self.scale, self.qk_norm, self.sink, self.rotate_values = float(scale), bool(qk_norm), sink, bool(rotate_values)
+        self.kv_from = None if kv_from is None else int(kv_from)
+        self.freqs = rotary_frequencies(rd, float(rot["base"]), rot.get("scaling") or None)
+        self.v_freqs = rotary_frequencies(vdim, float(rot["base"]), None) if rotate_values else None
+        self.out_cols = heads * vdim
+
+    def proj_rows(self) -> list:
+        rows = [(self.p + "q", self.heads * self.dk)]
+        if self.kv_from is None:
+            rows += [(self.p + "k", self.kv_heads * self.dk), (self.p + "v", self.kv_heads * self.dv)]
+        return rows
+
+    def extra_shapes(self) -> dict:
+        sh = {self.p + "o": (self.width, self.heads * self.dv)}
+        if self.qk_norm:
+            sh[self.p + "q.norm"] = (self.dk,)
+            if self.kv_from is None:
+                sh[self.p + "k.norm"] = (self.dk,)
+        if self.sink == "learned":
+            sh[self.p + "sink"] = (self.heads,)
+        return sh
+
+    def finish_weights(self, w: dict) -> None:
+        dev = w[self.p + "o"].device
+        self.freqs = self.freqs.to(dev)
+        if self.v_freqs is not None:
+            self.v_freqs = self.v_freqs.to(dev)
+        if self.sink == "learned":
+            _fp32(w, self.p + "sink")
+        elif self.sink == "zero":
+            w[self.p + "sink"] = torch.zeros(self.heads, dtype=torch.float32, device=dev)
+
+    def mix(self, parts: list, h: torch.Tensor, w: dict, ctx: StepContext, koff: int, voff: int, soff: int,
+            out: Optional[torch.Tensor] = None, out_scale: float = 1.0) -> torch.Tensor:
+        """The heads' outputs [T, H*dv] before the output projection (into `out`, times out_scale)."""
+        md, p = ctx.md, self.p
+        q = parts[0]
+        k, v = (parts[1], parts[2]) if self.kv_from is None else (None, None)
+        seqmix.rope_qkv_cache(q, k, v, md.positions, md.slot_mapping, ctx.cache, koff, voff, self.heads, self.kv_heads,
+                              self.dk, self.dv, ctx.block_size, self.freqs, w.get(p + "q.norm"), w.get(p + "k.norm"),
+                              ctx.eps, self.v_freqs)
+        o = seqmix.window_attention(q, ctx.cache, md.block_tables, md.query_start_loc, md.seq_lens, koff, voff,
+                                    self.heads, self.kv_heads, self.dk, self.dv, ctx.block_size, self.scale, 0, 0,
+                                    md.max_query_len, sink=w.get(p + "sink"))
+        if not self.rotate_values and out is None and out_scale == 1.0:
+            return o
+        if out is None:
+            out = torch.empty_like(o)
+        fr = self.v_freqs if self.rotate_values else self.freqs[:0]
+        seqmix.rope_rows(o, md.positions, self.heads, self.dv, fr, -1.0, out_scale, out)
+        return out
+
+    def forward(self, parts: list, h: torch.Tensor, w: dict, ctx: StepContext, koff: int, voff: int, soff: int):
+        return ops.linear(self.mix(parts, h, w, ctx, koff, voff, soff), w[self.p + "o"])
+
+
+class Mamba2(Mixer):
+    """in -> [z | x | B | C | dt]; x, B, C through a causal convolution with bias and SiLU; the scan;
+    y * SiLU(z), RMS norm in `norm_groups` slices, output projection.  State per sequence: the scan's
+    S [heads, vdim, state] and the convolution's last taps - 1 inputs."""
+
+    def __init__(self, prefix: str, width: int, heads: int, vdim: int, state: int, groups: int, conv: int,
+                 norm_groups: int):
+        inner = heads * vdim
+        if heads % groups or inner % norm_groups or conv < 1:
+            raise ValueError(f"{prefix}: heads {heads} / groups {groups} / norm_groups {norm_groups} do not divide")
+        self.p, self.width = prefix, width
+        self.heads, self.P, self.N, self.G, self.taps, self.norm_groups = heads, vdim, state, groups, conv, norm_groups
+        self.inner, self.conv_ch = inner, inner + 2 * groups * state
+        self.scan_floats = heads * vdim * state
+        self.state_floats = self.scan_floats + (conv - 1) * self.conv_ch
+        self.out_cols = inner
+
+    def proj_rows(self) -> list:
+        return [(self.p + "in", 2 * self.inner + 2 * self.G * self.N + self.heads)]
+
+    def extra_shapes(self) -> dict:
+        p, H = self.p, self.heads
+        return {p + "conv": (self.conv_ch, self.taps), p + "conv.b": (self.conv_ch,), p + "dt_bias": (H,),
+                p + "A_log": (H,), p + "D": (H,), p + "norm": (self.inner,), p + "o": (self.width, self.inner)}
+
+    def finish_weights(self, w: dict) -> None:
+        for n in ("dt_bias", "A_log", "D"):
+            _fp32(w, self.p + n)
+
+    def mix(self, parts: list, h: torch.Tensor, w: dict, ctx: StepContext, koff: int, voff: int, soff: int,
+            out: Optional[torch.Tensor] = None, out_scale: float = 1.0) -> torch.Tensor:
+        md, p = ctx.md, self.p
+        y = parts[0]
+        I, GN = self.inner, self.G * self.N
+        z, xbc, dt = y[:, :I], y[:, I:I + self.conv_ch], y[:, I + self.conv_ch:]
+        c = seqmix.causal_conv(xbc, w[p + "conv"], w[p + "conv.b"], ctx.state, md.state_rows, soff + self.scan_floats,
+                               md.query_start_loc, md.seq_lens, silu=True)
+        o = seqmix.ssd_scan(c[:, :I], c[:, I:I + GN], c[:, I + GN:], dt, w[p + "dt_bias"], w[p + "A_log"], w[p + "D"],
+                            ctx.state, md.state_rows, soff, md.query_start_loc, md.seq_lens, self.heads, self.G,
+                            self.N, self.P)
+        return seqmix.gated_norm(o, z, w[p + "norm"], ctx.eps, self.norm_groups, "silu", True, h.dtype, out_scale, out)
+
+    def forward(self, parts: list, h: torch.Tensor, w: dict, ctx: StepContext, koff: int, voff: int, soff: int):
+        return ops.linear(self.mix(parts, h, w, ctx, koff, voff, soff), w[self.p + "o"])
+
+
+class GatedDeltaRule(Mixer):
+    """q, k (qk_heads x dim) and v (heads x vdim) through short convolutions (no bias) and SiLU; q, k
+    unit vectors per head, q times dim^-1/2; write strength sigmoid(b h) per head; decay per head and
+    key channel from the low-rank pair a1, a2 with dt_bias and A_log; per-head RMS norm of the
+    read-out with a weight shared by the heads, times sigmoid of the low-rank gate g1, g2.  State per
+    sequence: S [heads, vdim, dim] and the three convolutions' last taps - 1 inputs (one block)."""
+
+    def __init__(self, prefix: str, width: int, heads: int, qk_heads: int, dim: int, vdim: int, conv: int,
+                 unit_eps: float = 1e-6):
+        if heads % qk_heads or conv < 1:
+            raise ValueError(f"{prefix}: {heads} heads do not divide over {qk_heads} q/k heads")
+        self.p, self.width = prefix, width
+        self.heads, self.G, self.dk, self.dv, self.taps = heads, qk_heads, dim, vdim, conv
+        self.unit_eps = float(unit_eps)
+        self.conv_ch = 2 * qk_heads * dim + heads * vdim
+        self.scan_floats = heads * vdim * dim
+        self.state_floats = self.scan_floats + (conv - 1) * self.conv_ch
+        # the low-rank pairs' inner sizes are no config entries: a checkpoint's tensors give them
+        # (adopt_shapes); these are what random weights are made with
+        self.rank_a = self.rank_g = 16
+        self.out_cols = heads * vdim
+
+    def adopt_shapes(self, full: dict) -> None:
+        a1, g1 = full.get(self.p + "a1"), full.get(self.p + "g1")
+        if a1 is not None and a1.dim() == 2:
+            self.rank_a = int(a1.shape[0])
+        if g1 is not None and g1.dim() == 2:
+            self.rank_g = int(g1.shape[0])
+
+    def proj_rows(self) -> list:
+        p, n = self.p, self.G * self.dk
+        return [(p + "q", n), (p + "k", n), (p + "v", self.heads * self.dv), (p + "a1", self.rank_a),
+                (p + "g1", self.rank_g), (p + "b", self.heads)]
+
+    def extra_shapes(self) -> dict:
+        p, H, n = self.p, self.heads, self.G * self.dk
+        return {p + "q.conv": (n, self.taps), p + "k.conv": (n, self.taps), p + "v.conv": (H * self.dv, self.taps),
+                p + "a2": (H * self.dk, self.rank_a), p + "g2": (H * self.dv, self.rank_g), p + "dt_bias": (H * self.dk,),
+                p + "A_log": (H,), p + "norm": (self.dv,), p + "o": (self.width, H * self.dv)}
+
+    def finish_weights(self, w: dict) -> None:
+        p = self.p
+        w[p + "_conv"] = torch.cat([w.pop(p + "q.conv"), w.pop(p + "k.conv"), w.pop(p + "v.conv")]).contiguous()
+        _fp32(w, p + "dt_bias")
+        _fp32(w, p + "A_log")
+
+    def mix(self, parts: list, h: torch.Tensor, w: dict, ctx: StepContext, koff: int, voff: int, soff: int,
+            out: Optional[torch.Tensor] = None, out_scale: float = 1.0) -> torch.Tensor:
+        md, p = ctx.md, self.p
+        q, k, v, a1, g1, b = parts
+        n = self.G * self.dk
+        # q, k, v are neighbours in the fused projection (proj_rows): one convolution over all their channels
+        qkv = torch.as_strided(q, (q.shape[0], self.conv_ch), q.stride(), q.storage_offset())
+        c = seqmix.causal_conv(qkv, w[p + "_conv"], None, ctx.state, md.state_rows, soff + self.scan_floats,
+                               md.query_start_loc, md.seq_lens, silu=True)
+        a = ops.linear(a1.contiguous(), w[p + "a2"])
+        g = ops.linear(g1.contiguous(), w[p + "g2"])
+        o = seqmix.delta_scan(c[:, :n], c[:, n:2 * n], c[:, 2 * n:], b, a, w[p + "dt_bias"], w[p + "A_log"], ctx.state,
+                              md.state_rows, soff, md.query_start_loc, md.seq_lens, self.heads, self.G, self.dk, self.dv,
+                              self.dk ** -0.5, self.unit_eps)
+        return seqmix.gated_norm(o, g, w[p + "norm"], ctx.eps, self.heads, "sigmoid", False, h.dtype, out_scale, out)
+
+    def forward(self, parts: list, h: torch.Tensor, w: dict, ctx: StepContext, koff: int, voff: int, soff: int):
+        return ops.linear(self.mix(parts, h, w, ctx, koff, voff, soff), w[self.p + "o"])
+
+
+class ScaledPair(Mixer):
+    """left_scale * left + right_scale * right.  Both output projections are one GEMM: each mixer
+    writes its activations, times its scale, into its columns of a shared buffer, and the two
+    projection weights stand side by side."""
+
+    def __init__(self, prefix: str, width: int, left: Mixer, right: Mixer, left_scale: float, right_scale: float):
+        if right.kv_heads:
+            raise ValueError("ScaledPair: only the left mixer may keep paged K/V")
+        if left.state_floats:
+            raise ValueError("ScaledPair: only the right mixer may keep a recurrent state")
+        self.p, self.width, self.left, self.right = prefix, width, left, right
+        self.ls, self.rs = float(left_scale), float(right_scale)
+        self.kv_heads, self.dk, self.dv = left.kv_heads, left.dk, left.dv
+        self.kv_from = getattr(left, "kv_from", None)
+        self.state_floats = right.state_floats
+
+    def proj_rows(self) -> list:
+        return self.left.proj_rows() + self.right.proj_rows()
+
+    def extra_shapes(self) -> dict:
+        return {**self.left.extra_shapes(), **self.right.extra_shapes()}
+
+    def adopt_shapes(self, full: dict) -> None:
+        for m in (self.left, self.right):
+            if hasattr(m, "adopt_shapes"):
+                m.adopt_shapes(full)
+
+    def finish_weights(self, w: dict) -> None:
+        for m in (self.left, self.right):
+            m.finish_weights(w)
+        w[self.p + "_o"] = torch.cat([w.pop(self.left.p + "o"), w.pop(self.right.p + "o")], dim=1).contiguous()
+
+    def forward(self, parts: list, h: torch.Tensor, w: dict, ctx: StepContext, koff: int, voff: int, soff: int):
+        nl, cl = len(self.left.proj_rows()), self.left.out_cols
+        buf = torch.empty(h.shape[0], cl + self.right.out_cols, dtype=h.dtype, device=h.device)
+        self.left.mix(parts[:nl], h, w, ctx, koff, voff, soff, out=buf[:, :cl], out_scale=self.ls)
+        self.right.mix(parts[nl:], h, w, ctx, koff, voff, soff, out=buf[:, cl:], out_scale=self.rs)
+        return ops.linear(buf, w[self.p + "_o"])
 
 
 def build_mixer(kind: str, prefix: str, width: int, mc: dict) -> Mixer:

@@ -12,7 +12,6 @@ for the recurrent mixers in the runner's per-request slots.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
 from typing import Optional
 
 import torch
@@ -20,38 +19,16 @@ import torch.nn.functional as F
 
 from .. import ops
 from ..ops import seqmix
-from ..parallel.comm import get_tp
 from .config import ModelConfig
+from .hybrid import HybridLM, LayerPlan, LayerRun, plan_runs  # noqa: F401  (LayerRun: part of this module's surface)
 from .mixers import Mixer, StepContext, build_mixer
 
 
-@dataclass
-class LayerRun:
-    """One execution of a layer: the looped span's layers appear once per pass."""
-    layer: int
-    loop_pass: Optional[int]  # pass number inside the looped span, None outside it
-    first_of_pass: bool
-    kv_heads: int = 0
-    dk: int = 0
-    dv: int = 0
-    koff: int = 0  # element offsets inside a cache block
-    voff: int = 0
-    soff: int = 0  # float offset inside a state slot
-
-
-@dataclass
-class LayerPlan:
-    runs: list = field(default_factory=list)
-    block_elems: int = 0  # K/V elements one block holds over all runs
-    state_floats: int = 0
-
-    @property
-    def attn_runs(self) -> list:
-        return [r for r in self.runs if r.kv_heads]
-
-
-def _mixers(ac: dict) -> list:
+def mixers_of(ac: dict) -> list:
     return [build_mixer(l["type"], f"l{i}.mix.", int(ac["width"]), l["mixer"]) for i, l in enumerate(ac["layers"])]
+
+
+_mixers = mixers_of
 
 
 def layer_plan(ac: dict, block_size: int = 16, mixers: Optional[list] = None) -> LayerPlan:
@@ -68,18 +45,7 @@ def layer_plan(ac: dict, block_size: int = 16, mixers: Optional[list] = None) ->
         for t in range(times):
             order += [(i, t, i == a) for i in range(a, b)]
         order += [(i, None, False) for i in range(b, n)]
-    plan = LayerPlan()
-    for i, t, first in order:
-        m: Mixer = mixers[i]
-        r = LayerRun(i, t, first, m.kv_heads, m.dk, m.dv)
-        if m.kv_heads:
-            r.koff = plan.block_elems
-            r.voff = r.koff + m.kv_heads * block_size * m.dk
-            plan.block_elems = r.voff + m.kv_heads * block_size * m.dv
-        r.soff = plan.state_floats
-        plan.state_floats += m.state_floats
-        plan.runs.append(r)
-    return plan
+    return plan_runs(order, mixers, block_size)
 
 
 def weight_shapes(ac: dict, mixers: Optional[list] = None) -> dict:
@@ -127,87 +93,16 @@ def random_state(ac: dict, seed: int = 0, device="cpu") -> dict:
     return out
 
 
-class VoletarLM:
-    """Same surface as TransformerLM for the model runner: weights in a flat dict, forward() over a
-    step's batch, compute_logits()."""
-
-    is_recurrent = True
+class VoletarLM(HybridLM):
+    """Voletar on the shared surface of the layer-list designs (mxserve/models/hybrid.py)."""
 
     def __init__(self, cfg: ModelConfig, device, dtype: torch.dtype = torch.bfloat16, block_size: int = 16):
-        if cfg.arch_config is None:
-            raise ValueError("VoletarLM needs the checkpoint's layer list (ModelConfig.arch_config)")
-        tp = get_tp()
-        if tp.tp_size != 1:
-            raise ValueError("Voletar runs on one GPU per replica (its recurrent state is not sharded)")
-        self.cfg, self.ac = cfg, cfg.arch_config
-        self.device, self.dtype = torch.device(device), dtype
-        self.tp_rank, self.tp_size = 0, 1
-        self.block_size = block_size
-        self.width = int(self.ac["width"])
-        self.eps = float(self.ac.get("norm", {}).get("eps", 1e-5))
+        import sys
+        self.design = sys.modules[__name__]
+        super().__init__(cfg, device, dtype, block_size)
         self.softcap = float(self.ac.get("logit_softcap") or 0.0)
-        self.mixers = _mixers(self.ac)
-        self.plan = layer_plan(self.ac, block_size, self.mixers)
-        self.state_floats = self.plan.state_floats
-        self.vocab_local = cfg.vocab_size
-        self.w: dict[str, torch.Tensor] = {}
-        self.kv_scales = [{"k_scale": 1.0, "v_scale": 1.0}]
-        self.pf_chain = False
-        # debugging tap: a list here receives the residual stream after every layer run (fp32 copies)
-        self.layer_tap: Optional[list] = None
-
-    # ------------------------------------------------------------------ cache / state geometry
-    def kv_cache_shape(self, num_blocks: int, block_size: int) -> tuple:
-        if block_size != self.block_size:
-            self.block_size = block_size
-            self.plan = layer_plan(self.ac, block_size, self.mixers)
-        return (num_blocks, max(self.plan.block_elems, 1))
-
-    # ------------------------------------------------------------------ weights
-    def init_random(self, seed: int = 0, std: float = 0.02) -> None:
-        self.load_full_state(random_state(self.ac, seed, device=self.device))
-
-    def load_full_state(self, full: dict) -> None:
-        """Checkpoint tensors (any float dtype; integer tables stay integers) -> this model's dtype, the
-        mixers' input projections concatenated into one weight per layer."""
-        shapes = weight_shapes(self.ac, self.mixers)
-        missing = [k for k in shapes if k not in full]
-        if missing:
-            raise KeyError(f"checkpoint lacks {missing[:4]}{' ...' if len(missing) > 4 else ''}")
-        w = {}
-        for name, shape in shapes.items():
-            t = full[name]
-            if tuple(t.shape) != tuple(shape):
-                raise ValueError(f"{name}: shape {tuple(t.shape)}, the config gives {tuple(shape)}")
-            w[name] = t.to(device=self.device, dtype=self.dtype if t.is_floating_point() else t.dtype).contiguous()
-        for i, m in enumerate(self.mixers):
-            rows = m.proj_rows()
-            w[f"l{i}.mix._in"] = torch.cat([w.pop(name) for name, _ in rows]).contiguous()
-            if hasattr(m, "finish_weights"):
-                m.finish_weights(w)
-        self.w = w
-
-    def prepare_fused_prefill(self, tuning: bool = True, max_rows: int = 8192) -> bool:
-        return False
-
-    def calibrate_kv_scales(self, block_size: int = 16, n: int = 256, headroom: float = 2.0) -> None:
-        raise ValueError("Voletar keeps its K/V pages in the model dtype (no fp8 KV cache)")
-
-    def lm_head_weight(self) -> torch.Tensor:
-        return self.w["head"]
-
-    def tunable_shapes(self) -> dict:
-        """Decode-GEMM shapes for the start-up tuner: none, the projections run hipBLASLt's own choice."""
-        return {}
 
     # ------------------------------------------------------------------ forward
-    def _split(self, y: torch.Tensor, mixer: Mixer) -> list:
-        parts, c = [], 0
-        for _, rows in mixer.proj_rows():
-            parts.append(y[:, c:c + rows])
-            c += rows
-        return parts
-
     def _add(self, x: torch.Tensor, pending, norm_w: Optional[torch.Tensor]):
         """Add a sublayer's output (a tensor, or the two branch outputs of a parallel mixer with their
         width norms) to the stream and return the next RMSNorm's output, if one is asked for."""

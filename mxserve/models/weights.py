@@ -182,7 +182,7 @@ def load_sharded_safetensors(model, model_dir: str) -> int:
 
 def load_weights(model, load_format: str = "auto", seed: int = 0) -> str:
     """Populate `model`.  Returns the source used: 'safetensors' | 'random'."""
-    if model.cfg.arch == "voletar":  # checkpoint names are the model's own (mxserve/models/voletar.py)
+    if model.cfg.arch_config is not None:  # layer-list designs: checkpoint names are the model's own
         model_dir = find_local_model_dir(model.cfg.name)
         files = sorted(glob.glob(os.path.join(model_dir, "*.safetensors"))) if model_dir else []
         if load_format in ("auto", "safetensors") and files:

@@ -14,7 +14,9 @@ position 0 starts from a zero state, whatever its slot held before.
 Paged cache of one attention layer inside the block-major pool `cache` [num_blocks, block_elems]:
 K at `koff` as [Hkv, BS, dk], V at `voff` as [Hkv, BS, dv], both token-major.
 Recurrent state of one layer inside the slot pool `state` [slots, state_floats] (fp32): decayed
-linear attention S [H, dk, dv] at `off`; mLSTM S [H, dk, dv], then n [H, dk], then m [H].
+linear attention S [H, dk, dv] at `off`; mLSTM S [H, dk, dv], then n [H, dk], then m [H]; the
+column scans (state-space duality, gated delta rule) S transposed [H, dv, dk], so that the rows a
+lane owns are contiguous; a short causal convolution its last taps - 1 inputs [taps - 1, channels].
 """
 from __future__ import annotations
 
@@ -163,18 +165,19 @@ def kv_write(cache: torch.Tensor, k: torch.Tensor, v: torch.Tensor, slot_mapping
 def window_attention(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor, qsl: torch.Tensor,
                      seq_lens: torch.Tensor, koff: int, voff: int, num_heads: int, num_kv_heads: int, dk: int,
                      dv: int, block_size: int, scale: float, window: int, keep_first: int,
-                     max_query_len: int = 0) -> torch.Tensor:
+                     max_query_len: int = 0, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Softmax attention over the paged cache (this step's keys already written).  The query at
     position i sees key j <= i when i - j < window or j < keep_first (window <= 0: every j <= i).
     q [T, H*dk] (row-strided view) -> [T, H*dv] in q's dtype; scores and weights in fp32.
-    Query head h reads kv head h // (H / Hkv).  max_query_len: the longest chunk of the step (host
+    Query head h reads kv head h // (H / Hkv).  sink (fp32 [H]): the softmax denominator of head h also
+    holds exp(sink[h]), a key without a value whose score is not scaled.  max_query_len: the longest chunk of the step (host
     int); from 16 rows a bf16 step with head sizes that are multiples of 16 runs the MFMA kernel."""
     T = q.shape[0]
     if _gpu(q):
         out = torch.empty(T, num_heads * dv, dtype=q.dtype, device=q.device)
         ext().window_attention(out, q, cache, block_tables, qsl, seq_lens, int(koff), int(voff), num_heads,
                                num_kv_heads, dk, dv, block_size, float(scale), int(window), int(keep_first),
-                               int(max_query_len))
+                               int(max_query_len), sink)
         return out
     out = torch.zeros(T, num_heads, dv, dtype=torch.float32)
     kc = cache[:, koff:koff + num_kv_heads * block_size * dk].view(-1, num_kv_heads, block_size, dk)
@@ -197,7 +200,10 @@ def window_attention(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.T
         seen = j <= i
         if window > 0:
             seen = seen & ((i - j < window) | (j < keep_first))
-        p = torch.softmax(sc.masked_fill(~seen.unsqueeze(0), float("-inf")), dim=-1)
+        sc = sc.masked_fill(~seen.unsqueeze(0), float("-inf"))
+        if sink is not None:  # one more column, dropped after the softmax: it has no value
+            sc = torch.cat([sc, sink.float().view(-1, 1, 1).expand(-1, sc.shape[1], 1)], dim=-1)
+        p = torch.softmax(sc, dim=-1)[..., :n]
         out[a:e] = torch.einsum("hmn,nhd->mhd", p, V.repeat_interleave(g, dim=1))
     return out.reshape(T, num_heads * dv).to(q.dtype)
 
@@ -313,3 +319,218 @@ def mlstm_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gates: torch.T
             den = torch.maximum((n * qf[t]).sum(-1).abs(), torch.exp(-m)) + 1e-6
             out[t] = torch.einsum("hdv,hd->hv", S, qf[t]) / den.unsqueeze(1)
     return out.reshape(T, H * dv)
+
+
+# ----------------------------------------------------------------------------- embedding, feed-forward
+def embed_scaled(ids: torch.Tensor, table: torch.Tensor, scale: float) -> torch.Tensor:
+    """table[ids] * scale as the fp32 residual stream [T, W]."""
+    if _gpu(table):
+        out = torch.empty(ids.shape[0], table.shape[1], dtype=torch.float32, device=table.device)
+        ext().embed_scaled(out, ids, table, float(scale))
+        return out
+    return F.embedding(ids, table).float() * scale
+
+
+def silu_mul(gu: torch.Tensor) -> torch.Tensor:
+    """SiLU(gu[:, :F]) * gu[:, F:] of a fused gate/up projection [T, 2F]; fp32 inside."""
+    Fh = gu.shape[1] // 2
+    if _gpu(gu):
+        out = torch.empty(gu.shape[0], Fh, dtype=gu.dtype, device=gu.device)
+        ext().silu_mul(out, gu)
+        return out
+    return (F.silu(gu[:, :Fh].float()) * gu[:, Fh:].float()).to(gu.dtype)
+
+
+# ----------------------------------------------------------------------------- rotary positions
+def _rotate(x: torch.Tensor, pos: torch.Tensor, freqs: torch.Tensor, sign: float) -> torch.Tensor:
+    """x fp32 [T, heads, dim]: pair (2i, 2i+1) turned by sign * pos * freqs[i]; the rest passes."""
+    n = freqs.numel()
+    ang = pos.to(torch.float32).view(-1, 1, 1) * freqs.float().view(1, 1, n) * sign
+    c, s = torch.cos(ang), torch.sin(ang)
+    u, v = x[..., 0:2 * n:2], x[..., 1:2 * n:2]
+    y = x.clone()
+    y[..., 0:2 * n:2] = u * c - v * s
+    y[..., 1:2 * n:2] = v * c + u * s
+    return y
+
+
+def rope_qkv_cache(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor], positions: torch.Tensor,
+                   slot_mapping: torch.Tensor, cache: torch.Tensor, koff: int, voff: int, num_heads: int,
+                   num_kv_heads: int, dk: int, dv: int, block_size: int, freqs: torch.Tensor,
+                   q_norm: Optional[torch.Tensor] = None, k_norm: Optional[torch.Tensor] = None, eps: float = 1e-5,
+                   v_freqs: Optional[torch.Tensor] = None) -> None:
+    """Queries, keys and values of a step from the fused projection to what attention reads, in one
+    launch.  Per head: optional RMS norm over the head (weight [dk], plain), then interleaved rotary
+    pairs (2i, 2i+1) on the first 2 * len(freqs) dimensions by position * freqs[i]; values are
+    turned over 2 * len(v_freqs) dimensions when v_freqs is given.  q [T, H*dk] is rewritten in place;
+    k [T, G*dk] and v [T, G*dv] go into the paged cache (slot -1: not written).  k = v = None: a layer
+    that reads another layer's pages.  Angles, norms and rotations in fp32, one rounding at the end."""
+    if _gpu(q):
+        ext().rope_qkv_cache(q, k, v, positions, slot_mapping, cache, int(koff), int(voff), num_heads, num_kv_heads,
+                             dk, dv, block_size, freqs, q_norm, k_norm, float(eps), v_freqs)
+        return
+    T = q.shape[0]
+
+    def prep(x, heads, dim, norm_w, fr):
+        y = x.float().reshape(T, heads, dim)
+        if norm_w is not None:
+            y = _rms(y, eps) * norm_w.float()
+        return _rotate(y, positions, fr, 1.0) if fr is not None else y
+
+    q.copy_(prep(q, num_heads, dk, q_norm, freqs).reshape(T, -1).to(q.dtype))
+    if k is None:
+        return
+    kk = prep(k, num_kv_heads, dk, k_norm, freqs).reshape(T, -1).to(k.dtype)
+    vv = prep(v, num_kv_heads, dv, None, v_freqs).reshape(T, -1).to(v.dtype)
+    kv_write(cache, kk, vv, slot_mapping, koff, voff, num_kv_heads, dk, dv, block_size)
+
+
+def rope_rows(x: torch.Tensor, positions: torch.Tensor, heads: int, dim: int, freqs: torch.Tensor, sign: float,
+              out_scale: float, out: torch.Tensor) -> None:
+    """out = out_scale * (x with every head's pairs (2i, 2i+1) turned by sign * position * freqs[i]).
+    x [T, heads*dim]; out may be a row-strided view of the same shape (a slice of a wider buffer)."""
+    if _gpu(x):
+        ext().rope_rows(out, x, positions, heads, dim, freqs, float(sign), float(out_scale))
+        return
+    T = x.shape[0]
+    out.copy_((_rotate(x.float().reshape(T, heads, dim), positions, freqs, sign) * out_scale).reshape(T, -1).to(out.dtype))
+
+
+# ----------------------------------------------------------------------------- short causal convolution
+def causal_conv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor,
+                state_rows: torch.Tensor, off: int, qsl: torch.Tensor, seq_lens: torch.Tensor,
+                silu: bool = True) -> torch.Tensor:
+    """Per-channel causal filter over time: y[t, c] = bias[c] + sum_j w[c, j] x[t - (taps-1) + j, c], the
+    last column of w weighing the current token, inputs before a sequence's start being zero; then
+    SiLU.  x [T, C] (row-strided view), w [C, taps].  The sequence's last taps - 1 inputs live in its
+    state slot at `off` as fp32 [taps - 1, C], oldest first, and are replaced by this step's."""
+    T, C = x.shape
+    taps = w.shape[1]
+    if _gpu(x):
+        out = torch.empty(T, C, dtype=x.dtype, device=x.device)
+        ext().causal_conv(out, x, w, bias, state, state_rows, int(off), qsl, seq_lens, bool(silu))
+        return out
+    out = torch.zeros(T, C, dtype=torch.float32)
+    ql, sl, rows = qsl.tolist(), seq_lens.tolist(), state_rows.tolist()
+    wf = w.float()
+    for s in range(len(sl)):
+        a, e = ql[s], ql[s + 1]
+        if e <= a:
+            continue
+        n = e - a
+        st = state[rows[s], off:off + (taps - 1) * C].view(taps - 1, C)
+        prev = torch.zeros(taps - 1, C) if sl[s] - n == 0 else st.clone()
+        full = torch.cat([prev, x[a:e].float()])
+        y = torch.zeros(n, C) if bias is None else bias.float().expand(n, C).clone()
+        for j in range(taps):
+            y += wf[:, j] * full[j:j + n]
+        out[a:e] = y
+        if taps > 1:
+            st.copy_(full[n:])
+    return (F.silu(out) if silu else out).to(x.dtype)
+
+
+# ----------------------------------------------------------------------------- column scans
+def ssd_scan(x: torch.Tensor, B: torch.Tensor, C: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor,
+             A_log: torch.Tensor, D: torch.Tensor, state: torch.Tensor, state_rows: torch.Tensor, off: int,
+             qsl: torch.Tensor, seq_lens: torch.Tensor, num_heads: int, groups: int, N: int, P: int) -> torch.Tensor:
+    """Selective state-space recurrence with a scalar decay per head and token (state-space duality):
+        d = softplus(dt + dt_bias_h);  S = exp(-exp(A_log_h) d) S + d B_g x_h^T;  y_h = S^T C_g + D_h x_h
+    with S [N, P] per head and head h reading group h // (H / G).  x [T, H*P], B, C [T, G*N], dt [T, H]
+    (row-strided views of any float dtype); dt_bias, A_log, D fp32 [H].  Returns y fp32 [T, H*P]; the
+    state (fp32, stored [H, P, N]) stays in the sequence's slot."""
+    T = x.shape[0]
+    H = num_heads
+    if _gpu(x):
+        out = torch.empty(T, H * P, dtype=torch.float32, device=x.device)
+        ext().ssd_scan(out, x, B, C, dt, dt_bias, A_log, D, state, state_rows, int(off), qsl, seq_lens, H, groups, N, P)
+        return out
+    out = torch.zeros(T, H, P, dtype=torch.float32)
+    xf = x.float().reshape(T, H, P)
+    rep = H // groups
+    Bf = B.float().reshape(T, groups, N).repeat_interleave(rep, dim=1)
+    Cf = C.float().reshape(T, groups, N).repeat_interleave(rep, dim=1)
+    d = F.softplus(dt.float() + dt_bias.float(), threshold=1e9)
+    a = torch.exp(-torch.exp(A_log.float()) * d)
+    ql, sl, rows = qsl.tolist(), seq_lens.tolist(), state_rows.tolist()
+    for s in range(len(sl)):
+        b, e = ql[s], ql[s + 1]
+        if e <= b:
+            continue
+        S = state[rows[s], off:off + H * P * N].view(H, P, N)
+        if sl[s] - (e - b) == 0:
+            S.zero_()
+        for t in range(b, e):
+            S.mul_(a[t].view(H, 1, 1)).add_((d[t].view(H, 1) * xf[t]).unsqueeze(2) * Bf[t].unsqueeze(1))
+            out[t] = (S * Cf[t].unsqueeze(1)).sum(-1) + D.float().view(H, 1) * xf[t]
+    return out.reshape(T, H * P)
+
+
+def delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, beta: torch.Tensor, a: torch.Tensor,
+               dt_bias: torch.Tensor, A_log: torch.Tensor, state: torch.Tensor, state_rows: torch.Tensor, off: int,
+               qsl: torch.Tensor, seq_lens: torch.Tensor, num_heads: int, qk_heads: int, dk: int, dv: int,
+               q_scale: float, unit_eps: float = 1e-6) -> torch.Tensor:
+    """Gated delta rule with one decay per head and key channel.  q, k [T, G*dk] are made unit vectors
+    per head (x / sqrt(sum x^2 + unit_eps)), q also times q_scale; head h reads q/k head h // (H / G).
+        g = exp(-exp(A_log_h) softplus(a + dt_bias))   [H, dk]      b = sigmoid(beta)   [H]
+        S = diag(g) S;   u = b (v - S^T k);   S = S + k u^T;   o = S^T q
+    so the read-out sees the token's own write.  v [T, H*dv], beta [T, H], a [T, H*dk] (row-strided
+    views); dt_bias fp32 [H*dk], A_log fp32 [H].  Returns o fp32 [T, H*dv]; S (fp32, stored [H, dv, dk])
+    stays in the sequence's slot."""
+    T = q.shape[0]
+    H, G = num_heads, qk_heads
+    if _gpu(q):
+        out = torch.empty(T, H * dv, dtype=torch.float32, device=q.device)
+        ext().delta_scan(out, q, k, v, beta, a, dt_bias, A_log, state, state_rows, int(off), qsl, seq_lens, H, G, dk,
+                         dv, float(q_scale), float(unit_eps))
+        return out
+    out = torch.zeros(T, H, dv, dtype=torch.float32)
+    rep = H // G
+
+    def unit(t):
+        t = t.float().reshape(T, G, dk)
+        return (t * torch.rsqrt(t.pow(2).sum(-1, keepdim=True) + unit_eps)).repeat_interleave(rep, dim=1)
+
+    qf, kf = unit(q) * q_scale, unit(k)
+    vf = v.float().reshape(T, H, dv)
+    b = torch.sigmoid(beta.float())
+    g = torch.exp(-torch.exp(A_log.float()).view(1, H, 1) *
+                  F.softplus(a.float() + dt_bias.float(), threshold=1e9).reshape(T, H, dk))
+    ql, sl, rows = qsl.tolist(), seq_lens.tolist(), state_rows.tolist()
+    for s in range(len(sl)):
+        c, e = ql[s], ql[s + 1]
+        if e <= c:
+            continue
+        S = state[rows[s], off:off + H * dv * dk].view(H, dv, dk)
+        if sl[s] - (e - c) == 0:
+            S.zero_()
+        for t in range(c, e):
+            S.mul_(g[t].unsqueeze(1))
+            u = b[t].view(H, 1) * (vf[t] - (S * kf[t].unsqueeze(1)).sum(-1))
+            S.add_(u.unsqueeze(2) * kf[t].unsqueeze(1))
+            out[t] = (S * qf[t].unsqueeze(1)).sum(-1)
+    return out.reshape(T, H * dv)
+
+
+def gated_norm(o: torch.Tensor, gate: torch.Tensor, w: torch.Tensor, eps: float, groups: int, act: str,
+               gate_first: bool, out_dtype: torch.dtype, out_scale: float = 1.0,
+               out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """A mixer's output norm with its gate.  o fp32 [T, N]; the RMS norm runs over each of `groups`
+    equal slices of a row; w has N entries or a divisor of N (then it repeats, e.g. one weight per
+    head size shared by the heads); act(gate) with act in silu | sigmoid multiplies before the norm
+    (gate_first) or after it.  The result, times out_scale, goes to `out` (may be a row-strided view
+    of a wider buffer) or a new [T, N] tensor of out_dtype."""
+    T, N = o.shape
+    if out is None:
+        out = torch.empty(T, N, dtype=out_dtype, device=o.device)
+    if _gpu(o):
+        ext().gated_norm(out, o, gate, w, float(eps), int(groups), act == "silu", bool(gate_first), float(out_scale))
+        return out
+    gf = F.silu(gate.float()) if act == "silu" else torch.sigmoid(gate.float())
+    wf = w.float().repeat(N // w.numel())
+    y = o * gf if gate_first else o
+    y = _rms(y.view(T, groups, N // groups), eps).reshape(T, N) * wf
+    if not gate_first:
+        y = y * gf
+    out.copy_((y * out_scale).to(out.dtype))
+    return out
