@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <torch/extension.h>
 
+#include "column_scan.h"
+
 namespace mxs {
 void launch_resid_update(float*, const void*, long, const void*, const void*, long, const void*, const void*, int,
                          const void*, void*, int, int, float, bool, hipStream_t);
@@ -16,10 +18,22 @@ void launch_gate_linear(float*, const void*, long, const void*, const void*, int
 void launch_kv_write(void*, long, const void*, long, const void*, long, const int64_t*, int, int, int, int, int, int,
                      int, bool, hipStream_t);
 bool launch_window_attention(void*, const void*, long, const void*, long, const int*, int, const int*, const int*, int,
-                             int, int, int, int, int, int, int, int, float, int, int, int, bool, hipStream_t);
+                             int, int, int, int, int, int, int, int, float, int, int, int, const float*, bool, hipStream_t);
 bool launch_matrix_scan(float*, const void*, long, const void*, long, const void*, long, const float*, const float*,
                         float*, long, const int*, long, const int*, const int*, int, int, int, int, int, int, float,
                         float, bool, bool, int, int, float*, float*, long, hipStream_t);
+void launch_embed_scaled(float*, const int64_t*, const void*, int, int, long, float, bool, hipStream_t);
+void launch_silu_mul(void*, const void*, long, int, int, bool, hipStream_t);
+void launch_rope_qkv_cache(void*, long, const void*, long, const void*, long, const int64_t*, const int64_t*, void*, long,
+                           int, int, int, int, int, int, int, int, const float*, int, const void*, const void*, float,
+                           const float*, int, bool, hipStream_t);
+void launch_rope_rows(void*, long, const void*, long, const int64_t*, int, int, int, const float*, int, float, float, bool,
+                      hipStream_t);
+void launch_causal_conv(void*, const void*, long, const void*, const void*, float*, long, const int*, long, const int*,
+                        const int*, int, int, int, int, int, bool, hipStream_t);
+void launch_gated_norm(void*, long, const float*, const void*, long, const void*, int, int, int, int, float, int, int,
+                       float, bool, hipStream_t);
+bool launch_column_scan(const ScanArgs&, int, bool, bool, hipStream_t);
 }  // namespace mxs
 
 namespace {
@@ -153,8 +167,13 @@ void kv_write(at::Tensor cache, at::Tensor k, at::Tensor v, at::Tensor slots, in
 
 void window_attention(at::Tensor out, at::Tensor q, at::Tensor cache, at::Tensor block_tables, at::Tensor qsl,
                       at::Tensor seq_lens, int64_t koff, int64_t voff, int64_t H, int64_t G, int64_t dk, int64_t dv,
-                      int64_t bs, double scale, int64_t window, int64_t keep, int64_t max_query_len) {
+                      int64_t bs, double scale, int64_t window, int64_t keep, int64_t max_query_len, OptT sink) {
   const bool bf = is_bf(q);
+  const float* sinkp = nullptr;
+  if (sink.has_value()) {
+    sinkp = f32(*sink, "sink");
+    TORCH_CHECK(sink->numel() == H, "sink: fp32 [H]");
+  }
   const int64_t T = q.size(0), S = seq_lens.numel();
   check_cache(cache, bf, koff, voff, G, dk, dv, bs);
   TORCH_CHECK(G >= 1 && H % G == 0, "query heads must divide over kv heads");
@@ -168,7 +187,7 @@ void window_attention(at::Tensor out, at::Tensor q, at::Tensor cache, at::Tensor
       i32(seq_lens, S, "seq_lens"), static_cast<int>(S), static_cast<int>(T), static_cast<int>(koff),
       static_cast<int>(voff), static_cast<int>(H), static_cast<int>(G), static_cast<int>(dk), static_cast<int>(dv),
       static_cast<int>(bs), static_cast<float>(scale), static_cast<int>(window), static_cast<int>(keep),
-      static_cast<int>(std::min<int64_t>(max_query_len, T)), bf, stream());
+      static_cast<int>(std::min<int64_t>(max_query_len, T)), sinkp, bf, stream());
   TORCH_CHECK(ok, "window_attention: head sizes beyond what the kernel holds (dv <= 512)");
 }
 
@@ -221,6 +240,159 @@ void mlstm_scan(at::Tensor out, at::Tensor q, at::Tensor k, at::Tensor v, at::Te
        q_scale, piece, npieces, sc_local, sc_start);
 }
 
+// ---- rotary attention, convolutions, column scans
+const int64_t* i64(const at::Tensor& t, int64_t n, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kLong && t.is_contiguous() && t.numel() == n, name,
+              ": expected ", n, " contiguous int64");
+  return t.data_ptr<int64_t>();
+}
+
+const float* f32n(const OptT& t, int64_t n, const char* name) {
+  if (!t.has_value()) return nullptr;
+  TORCH_CHECK(t->numel() == n, name, ": expected ", n, " elements");
+  return f32(*t, name);
+}
+
+void embed_scaled(at::Tensor out, at::Tensor ids, at::Tensor table, double scale) {
+  float* op = f32(out, "out");
+  TORCH_CHECK(table.is_cuda() && table.dim() == 2 && table.is_contiguous(), "table: contiguous [vocab, W]");
+  const int64_t T = ids.numel(), W = table.size(1);
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) == W, "out: fp32 [T, W]");
+  mxs::launch_embed_scaled(op, i64(ids, T, "ids"), table.data_ptr(), static_cast<int>(T), static_cast<int>(W),
+                           table.size(0), static_cast<float>(scale), is_bf(table), stream());
+}
+
+void silu_mul(at::Tensor out, at::Tensor gu) {
+  const bool bf = is_bf(gu);
+  TORCH_CHECK(gu.is_cuda() && gu.dim() == 2 && gu.stride(1) == 1 && gu.size(1) % 2 == 0, "gu: [T, 2F] with contiguous rows");
+  const int64_t T = gu.size(0), F = gu.size(1) / 2;
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.dim() == 2 && out.size(0) == T && out.size(1) == F &&
+              is_bf(out) == bf, "out: [T, F]");
+  mxs::launch_silu_mul(out.data_ptr(), gu.data_ptr(), gu.stride(0), static_cast<int>(T), static_cast<int>(F), bf, stream());
+}
+
+void rope_qkv_cache(at::Tensor q, OptT k, OptT v, at::Tensor positions, at::Tensor slots, at::Tensor cache, int64_t koff,
+                    int64_t voff, int64_t H, int64_t G, int64_t dk, int64_t dv, int64_t bs, at::Tensor freqs, OptT q_norm,
+                    OptT k_norm, double eps, OptT v_freqs) {
+  const bool bf = is_bf(q);
+  const int64_t T = q.size(0);
+  TORCH_CHECK(k.has_value() == v.has_value(), "k and v go together");
+  const void *kp = nullptr, *vp = nullptr;
+  if (k.has_value()) {
+    check_cache(cache, bf, koff, voff, G, dk, dv, bs);
+    kp = mat(*k, bf, T, G * dk, "k");
+    vp = mat(*v, bf, T, G * dv, "v");
+  }
+  const int64_t nf = freqs.numel(), nvf = v_freqs.has_value() ? v_freqs->numel() : 0;
+  TORCH_CHECK(2 * nf <= dk && 2 * nvf <= dv, "more rotary pairs than the head has dimensions");
+  mxs::launch_rope_qkv_cache(const_cast<void*>(mat(q, bf, T, H * dk, "q")), q.stride(0), kp, k.has_value() ? k->stride(0) : 0,
+                             vp, v.has_value() ? v->stride(0) : 0, i64(positions, T, "positions"),
+                             i64(slots, T, "slot_mapping"), cache.data_ptr(), cache.stride(0), static_cast<int>(T),
+                             static_cast<int>(koff), static_cast<int>(voff), static_cast<int>(H), static_cast<int>(G),
+                             static_cast<int>(dk), static_cast<int>(dv), static_cast<int>(bs), f32(freqs, "freqs"),
+                             static_cast<int>(nf), vec(q_norm, bf, dk, "q_norm"), vec(k_norm, bf, dk, "k_norm"),
+                             static_cast<float>(eps), f32n(v_freqs, nvf, "v_freqs"), static_cast<int>(nvf), bf, stream());
+}
+
+void rope_rows(at::Tensor out, at::Tensor x, at::Tensor positions, int64_t heads, int64_t dim, at::Tensor freqs,
+               double sign, double scale) {
+  const bool bf = is_bf(x);
+  const int64_t T = x.size(0);
+  TORCH_CHECK(2 * freqs.numel() <= dim, "more rotary pairs than the head has dimensions");
+  mxs::launch_rope_rows(const_cast<void*>(mat(out, bf, T, heads * dim, "out")), out.stride(0), mat(x, bf, T, heads * dim, "x"),
+                        x.stride(0), i64(positions, T, "positions"), static_cast<int>(T), static_cast<int>(heads),
+                        static_cast<int>(dim), f32(freqs, "freqs"), static_cast<int>(freqs.numel()),
+                        static_cast<float>(sign), static_cast<float>(scale), bf, stream());
+}
+
+void causal_conv(at::Tensor out, at::Tensor x, at::Tensor w, OptT bias, at::Tensor state, at::Tensor state_rows,
+                 int64_t off, at::Tensor qsl, at::Tensor seq_lens, bool silu) {
+  const bool bf = is_bf(x);
+  TORCH_CHECK(x.dim() == 2 && w.dim() == 2 && w.is_cuda() && w.is_contiguous() && is_bf(w) == bf && w.size(0) == x.size(1),
+              "causal_conv: x [T, C], w [C, taps] of one dtype");
+  const int64_t T = x.size(0), C = x.size(1), taps = w.size(1), S = seq_lens.numel();
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.dim() == 2 && out.size(0) == T && out.size(1) == C &&
+              is_bf(out) == bf, "out: contiguous [T, C]");
+  float* sp = f32(state, "state");
+  TORCH_CHECK(state.dim() == 2 && off >= 0 && off + (taps - 1) * C <= state.size(1), "state slot too small for this filter");
+  mxs::launch_causal_conv(out.data_ptr(), mat(x, bf, T, C, "x"), x.stride(0), w.data_ptr(), vec(bias, bf, C, "bias"), sp,
+                          state.stride(0), i32(state_rows, S, "state_rows"), off, i32(qsl, S + 1, "qsl"),
+                          i32(seq_lens, S, "seq_lens"), static_cast<int>(S), static_cast<int>(T), static_cast<int>(C),
+                          static_cast<int>(taps), silu ? 1 : 0, bf, stream());
+}
+
+void gated_norm(at::Tensor out, at::Tensor o, at::Tensor gate, at::Tensor w, double eps, int64_t groups, bool silu,
+                bool gate_first, double scale) {
+  const float* opn = f32(o, "o");
+  TORCH_CHECK(o.dim() == 2, "o: [T, N]");
+  const int64_t T = o.size(0), N = o.size(1), wn = w.numel();
+  const bool bf = is_bf(out);
+  TORCH_CHECK(groups >= 1 && N % groups == 0 && wn >= 1 && N % wn == 0, "groups and the weight's length must divide N");
+  mxs::launch_gated_norm(const_cast<void*>(mat(out, bf, T, N, "out")), out.stride(0), opn, mat(gate, bf, T, N, "gate"),
+                         gate.stride(0), vec(OptT(w), bf, wn, "w"), static_cast<int>(wn), static_cast<int>(T),
+                         static_cast<int>(N), static_cast<int>(groups), static_cast<float>(eps), silu ? 1 : 0,
+                         gate_first ? 1 : 0, static_cast<float>(scale), bf, stream());
+}
+
+void column_scan(bool delta, at::Tensor out, at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor beta, OptT a,
+                 at::Tensor dt_bias, at::Tensor A_log, OptT D, at::Tensor state, at::Tensor state_rows, int64_t off,
+                 at::Tensor qsl, at::Tensor seq_lens, int64_t H, int64_t G, int64_t dk, int64_t dv, double q_scale,
+                 double unit_eps) {
+  const bool bf = is_bf(q);
+  const int64_t T = q.size(0), S = seq_lens.numel();
+  TORCH_CHECK(G >= 1 && H % G == 0, "heads must divide over the q/k heads (groups)");
+  mxs::ScanArgs p{};
+  p.out = f32(out, "out");
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) == H * dv, "out: fp32 [T, H*dv]");
+  p.q = mat(q, bf, T, G * dk, "q");
+  p.q_stride = q.stride(0);
+  p.k = mat(k, bf, T, G * dk, "k");
+  p.k_stride = k.stride(0);
+  p.v = mat(v, bf, T, H * dv, "v");
+  p.v_stride = v.stride(0);
+  p.beta = mat(beta, bf, T, H, "beta");
+  p.beta_stride = beta.stride(0);
+  if (delta) {
+    TORCH_CHECK(a.has_value(), "the delta rule needs its decay pre-activations");
+    p.a = mat(*a, bf, T, H * dk, "a");
+    p.a_stride = a->stride(0);
+  } else {
+    TORCH_CHECK(D.has_value(), "the state-space scan needs D");
+  }
+  p.dt_bias = f32n(OptT(dt_bias), delta ? H * dk : H, "dt_bias");
+  p.A_log = f32n(OptT(A_log), H, "A_log");
+  p.D = f32n(D, H, "D");
+  p.state = f32(state, "state");
+  TORCH_CHECK(state.dim() == 2 && off >= 0 && off + H * dk * dv <= state.size(1), "state slot too small for this layer");
+  p.state_stride = state.stride(0);
+  p.state_rows = i32(state_rows, S, "state_rows");
+  p.off = off;
+  p.qsl = i32(qsl, S + 1, "qsl");
+  p.seq_lens = i32(seq_lens, S, "seq_lens");
+  p.n_rows = static_cast<int>(T);
+  p.H = static_cast<int>(H);
+  p.G = static_cast<int>(G);
+  p.dk = static_cast<int>(dk);
+  p.dv = static_cast<int>(dv);
+  p.q_scale = static_cast<float>(q_scale);
+  p.unit_eps = static_cast<float>(unit_eps);
+  TORCH_CHECK(mxs::launch_column_scan(p, static_cast<int>(S), delta, bf, stream()), "column scan: key / state size beyond 256");
+}
+
+void ssd_scan(at::Tensor out, at::Tensor x, at::Tensor B, at::Tensor C, at::Tensor dt, at::Tensor dt_bias, at::Tensor A_log,
+              at::Tensor D, at::Tensor state, at::Tensor state_rows, int64_t off, at::Tensor qsl, at::Tensor seq_lens,
+              int64_t H, int64_t G, int64_t N, int64_t P) {
+  column_scan(false, out, C, B, x, dt, OptT(), dt_bias, A_log, OptT(D), state, state_rows, off, qsl, seq_lens, H, G, N, P,
+              1.0, 0.0);
+}
+
+void delta_scan(at::Tensor out, at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor beta, at::Tensor a, at::Tensor dt_bias,
+                at::Tensor A_log, at::Tensor state, at::Tensor state_rows, int64_t off, at::Tensor qsl, at::Tensor seq_lens,
+                int64_t H, int64_t G, int64_t dk, int64_t dv, double q_scale, double unit_eps) {
+  column_scan(true, out, q, k, v, beta, OptT(a), dt_bias, A_log, OptT(), state, state_rows, off, qsl, seq_lens, H, G, dk, dv,
+              q_scale, unit_eps);
+}
+
 }  // namespace
 
 PYBIND11_MODULE(_M, m) {
@@ -234,4 +406,12 @@ PYBIND11_MODULE(_M, m) {
   m.def("window_attention", &window_attention);
   m.def("decay_scan", &decay_scan);
   m.def("mlstm_scan", &mlstm_scan);
+  m.def("embed_scaled", &embed_scaled);
+  m.def("silu_mul", &silu_mul);
+  m.def("rope_qkv_cache", &rope_qkv_cache);
+  m.def("rope_rows", &rope_rows);
+  m.def("causal_conv", &causal_conv);
+  m.def("gated_norm", &gated_norm);
+  m.def("ssd_scan", &ssd_scan);
+  m.def("delta_scan", &delta_scan);
 }

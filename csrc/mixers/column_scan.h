@@ -1,0 +1,31 @@
+// Arguments of the column scans (csrc/mixers/column_scan.hip), shared with the torch bindings.
+#pragma once
+
+namespace mxs {
+
+struct ScanArgs {
+  float* out;          // [T, H*dv]
+  const void* q;       // delta rule: queries [T, G*dk]; state space: C [T, G*dk]
+  long q_stride;
+  const void* k;       // delta rule: keys; state space: B
+  long k_stride;
+  const void* v;       // delta rule: values [T, H*dv]; state space: x
+  long v_stride;
+  const void* beta;    // delta rule: write strength before the sigmoid [T, H]; state space: dt before the softplus [T, H]
+  long beta_stride;
+  const void* a;       // delta rule: decay pre-activation [T, H*dk]
+  long a_stride;
+  const float* dt_bias;  // delta rule: [H*dk]; state space: [H]
+  const float* A_log;    // [H]
+  const float* D;        // state space: [H]
+  float* state;          // [slots, state_stride], this layer's S at `off` as [H][dv][dk]
+  long state_stride;
+  const int* state_rows;
+  long off;
+  const int* qsl;
+  const int* seq_lens;
+  int n_rows, H, G, dk, dv;
+  float q_scale, unit_eps;
+};
+
+}  // namespace mxs

@@ -5,6 +5,8 @@
 // query with the key's cache row), a block-wide running maximum and sum (online softmax), then each
 // wave takes every fourth key of the tile with its lanes across the value row.  Scores, weights and
 // the output sum are fp32; q, K and V are bf16 or fp32.
+// A sink (fp32 [H], optional) is one more key per head with the score sink[h], not scaled, and no
+// value: the running maximum starts at it and the running sum at 1 instead of -inf and 0.
 #include "mix_common.h"
 
 namespace mxs {
@@ -16,7 +18,8 @@ template <typename T>
 __global__ void __launch_bounds__(256) window_attention_kernel(
     T* __restrict__ out, const T* __restrict__ q, long q_stride, const T* __restrict__ cache, long block_stride,
     const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ qsl, const int* __restrict__ seq_lens,
-    int S, int koff, int voff, int H, int G, int dk, int dv, int bs, float scale, int window, int keep, bool vec) {
+    int S, int koff, int voff, int H, int G, int dk, int dv, int bs, float scale, int window, int keep, bool vec,
+    const float* __restrict__ sink) {
   extern __shared__ float lds[];
   float* qs = lds;                      // [dk]
   float* p = qs + ((dk + 3) & ~3);      // [kKeyTile]
@@ -34,7 +37,7 @@ __global__ void __launch_bounds__(256) window_attention_kernel(
   const int nvis = nA + (pos - lo + 1);
   const int* bt = block_tables + static_cast<long>(s) * bt_stride;
   for (int d = tid; d < dk; d += blockDim.x) qs[d] = ldf(q + static_cast<long>(t) * q_stride + hd * dk + d) * scale;
-  float m = -INFINITY, l = 0.f;
+  float m = sink ? sink[hd] : -INFINITY, l = sink ? 1.f : 0.f;
   float acc[kMaxVChunks];
 #pragma unroll
   for (int c = 0; c < kMaxVChunks; ++c) acc[c] = 0.f;
@@ -110,7 +113,8 @@ template <typename T, int NC, int RM>
 __global__ void __launch_bounds__(256) window_attention_rows_kernel(
     T* __restrict__ out, const T* __restrict__ q, long q_stride, const T* __restrict__ cache, long block_stride,
     const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ qsl, const int* __restrict__ seq_lens,
-    int S, int koff, int voff, int H, int G, int dk, int dv, int bs, float scale, int window, int keep, int nsplit) {
+    int S, int koff, int voff, int H, int G, int dk, int dv, int bs, float scale, int window, int keep, int nsplit,
+    const float* __restrict__ sink) {
   constexpr int EL = El<T>::N;
   extern __shared__ float lds[];
   float* p = lds;                      // [RM][kKeyTile]
@@ -133,8 +137,8 @@ __global__ void __launch_bounds__(256) window_attention_rows_kernel(
   float qf[RM][NC][EL], acc[RM][NC][EL], m[RM], l[RM];
 #pragma unroll
   for (int r = 0; r < RM; ++r) {
-    m[r] = -INFINITY;
-    l[r] = 0.f;
+    m[r] = (sink && r < nr) ? sink[h0 + r] : -INFINITY;
+    l[r] = (sink && r < nr) ? 1.f : 0.f;
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
       const int d = (c * 8 + part) * EL;
@@ -277,7 +281,7 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ cache,
     long block_stride, const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ qsl,
     const int* __restrict__ seq_lens, int koff, int voff, int H, int G, int dk, int dv, float scale, int window,
-    int keep) {
+    int keep, const float* __restrict__ sink) {
   // each wave's own staging area for a block's value rows (token-major in the pages): written with
   // 16-byte pieces, read back as the key-contiguous V^T operand.  Rows are padded by 8 elements so
   // that the four key groups of a read fall into different banks.
@@ -308,7 +312,9 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(
   const int lo_first = window > 0 ? max(pos0 - window + 1, 0) : 0;
   const int wb = lo_first >> 4, lastb = p_last >> 4;
   const int kA = window > 0 ? min((keep + 15) >> 4, wb) : 0;  // kept first blocks below the window's
-  float m = -INFINITY, l = 0.f;  // m in log2 units: scores are scaled by scale * log2(e), weights are exp2
+  // m in log2 units: scores are scaled by scale * log2(e), weights are exp2.  l is a lane's share of the
+  // row's sum (its key group's), added up at the end: the sink's 1 goes to the first group.
+  float m = sink ? sink[hd] * 1.4426950408889634f : -INFINITY, l = (sink && kg == 0) ? 1.f : 0.f;
   f4_t o[VTM];
 #pragma unroll
   for (int vt = 0; vt < VTM; ++vt) o[vt] = f4_t{0.f, 0.f, 0.f, 0.f};
@@ -409,7 +415,7 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(
 bool launch_window_attention(void* out, const void* q, long q_stride, const void* cache, long block_stride,
                              const int* block_tables, int bt_stride, const int* qsl, const int* seq_lens, int S,
                              int rows, int koff, int voff, int H, int G, int dk, int dv, int bs, float scale,
-                             int window, int keep, int max_q, bool bf, hipStream_t st) {
+                             int window, int keep, int max_q, const float* sink, bool bf, hipStream_t st) {
   if (rows == 0 || S == 0) return true;
   // prompt chunks in bf16 with MFMA-shaped heads: the matrix-core form (rows of a mixed step's single
   // tokens ride along as 1-row tiles); everything else the scalar form below
@@ -419,7 +425,7 @@ bool launch_window_attention(void* out, const void* q, long q_stride, const void
 #define MIX_WA(KSM, VTM)                                                                                              \
   hipLaunchKernelGGL((window_attention_mfma_kernel<KSM, VTM>), grid, dim3(256), 0, st, (bf16_t*)out, (const bf16_t*)q, \
                      q_stride, (const bf16_t*)cache, block_stride, block_tables, bt_stride, qsl, seq_lens, koff, voff, \
-                     H, G, dk, dv, scale, window, keep)
+                     H, G, dk, dv, scale, window, keep, sink)
     if (dk <= 64 && dv <= 64) MIX_WA(4, 4);
     else MIX_WA(8, 8);
 #undef MIX_WA
@@ -440,7 +446,7 @@ bool launch_window_attention(void* out, const void* q, long q_stride, const void
     const size_t sh = (static_cast<size_t>(RM) * kKeyTile + 4 * RM * dv) * sizeof(float);                             \
     hipLaunchKernelGGL((window_attention_rows_kernel<TT, NC, RM>), dim3(rows, G * nsplit), dim3(256), sh, st, (TT*)out, \
                        (const TT*)q, q_stride, (const TT*)cache, block_stride, block_tables, bt_stride, qsl, seq_lens, \
-                       S, koff, voff, H, G, dk, dv, bs, scale, window, keep, nsplit);                                  \
+                       S, koff, voff, H, G, dk, dv, bs, scale, window, keep, nsplit, sink);                            \
   } while (0)
 #define MIX_ROWS_T(TT)                                          \
   do {                                                          \
@@ -459,11 +465,11 @@ bool launch_window_attention(void* out, const void* q, long q_stride, const void
   if (bf)
     hipLaunchKernelGGL(window_attention_kernel<bf16_t>, dim3(rows, H), dim3(256), shm, st, (bf16_t*)out, (const bf16_t*)q,
                        q_stride, (const bf16_t*)cache, block_stride, block_tables, bt_stride, qsl, seq_lens, S, koff,
-                       voff, H, G, dk, dv, bs, scale, window, keep, vec);
+                       voff, H, G, dk, dv, bs, scale, window, keep, vec, sink);
   else
     hipLaunchKernelGGL(window_attention_kernel<float>, dim3(rows, H), dim3(256), shm, st, (float*)out, (const float*)q,
                        q_stride, (const float*)cache, block_stride, block_tables, bt_stride, qsl, seq_lens, S, koff,
-                       voff, H, G, dk, dv, bs, scale, window, keep, vec);
+                       voff, H, G, dk, dv, bs, scale, window, keep, vec, sink);
   MXS_CHECK_LAUNCH();
   return true;
 }
