@@ -99,16 +99,18 @@ def vlog(msg: str) -> None:
 def parse(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    # a separate measurement, not the headline: Voletar beside a Llama-shaped model of equal size
-    # (mxserve/tools/mixer_bench.py); without this flag nothing of the default workload changes
+    # a separate measurement, not the headline: a layer-list design beside the models closest to it at
+    # equal size (mxserve/tools/mixer_bench.py); without this flag nothing of the default workload changes
     ap.add_argument("--mixer-bench", action="store_true",
-                    help="prefill / decode throughput of Voletar beside a Llama-shaped model of equal size, and the "
-                         "mixer kernels against their rooflines; prints JSON lines and exits")
+                    help="prefill / decode throughput of Voletar (or, with --mixer-design tapasun, of Tapasun beside "
+                         "Voletar) and a Llama-shaped model of equal size, and the mixer kernels against their "
+                         "rooflines; prints JSON lines and exits")
+    ap.add_argument("--mixer-design", choices=["voletar", "tapasun"], default="voletar")
     ap.add_argument("--mixer-sizes", default="1024,2048", help="model widths, comma-separated")
     ap.add_argument("--mixer-prompt", type=int, default=4096)
     ap.add_argument("--mixer-batch", type=int, default=64)
     ap.add_argument("--mixer-context", type=int, default=2048)
-    ap.add_argument("--mixer-only", choices=["all", "voletar", "llama", "kernels"], default="all")
+    ap.add_argument("--mixer-only", choices=["all", "tapasun", "voletar", "llama", "kernels"], default="all")
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--iters-per-step", type=int, default=int(os.environ.get("MXS_BENCH_ITERS_PER_STEP", "50")),
@@ -1021,7 +1023,7 @@ def main():
     if a.mixer_bench:
         from mxserve.tools.mixer_bench import main as mixer_main
         return mixer_main([int(x) for x in a.mixer_sizes.split(",")], a.mixer_prompt, a.mixer_batch, a.mixer_context,
-                          only=a.mixer_only)
+                          only=a.mixer_only, design=a.mixer_design)
     world_env = os.environ.get("WORLD_SIZE")
     if world_env is None and a.gpus > 1:
         return launch_ranks(a)

@@ -308,9 +308,9 @@ void rope_rows(at::Tensor out, at::Tensor x, at::Tensor positions, int64_t heads
 void causal_conv(at::Tensor out, at::Tensor x, at::Tensor w, OptT bias, at::Tensor state, at::Tensor state_rows,
                  int64_t off, at::Tensor qsl, at::Tensor seq_lens, bool silu) {
   const bool bf = is_bf(x);
-  TORCH_CHECK(x.dim() == 2 && w.dim() == 2 && w.is_cuda() && w.is_contiguous() && is_bf(w) == bf && w.size(0) == x.size(1),
-              "causal_conv: x [T, C], w [C, taps] of one dtype");
-  const int64_t T = x.size(0), C = x.size(1), taps = w.size(1), S = seq_lens.numel();
+  TORCH_CHECK(x.dim() == 2 && w.dim() == 2 && w.is_cuda() && w.is_contiguous() && is_bf(w) == bf && w.size(1) == x.size(1),
+              "causal_conv: x [T, C], w [taps, C] of one dtype");
+  const int64_t T = x.size(0), C = x.size(1), taps = w.size(0), S = seq_lens.numel();
   TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.dim() == 2 && out.size(0) == T && out.size(1) == C &&
               is_bf(out) == bf, "out: contiguous [T, C]");
   float* sp = f32(state, "state");
@@ -337,7 +337,8 @@ void gated_norm(at::Tensor out, at::Tensor o, at::Tensor gate, at::Tensor w, dou
 void column_scan(bool delta, at::Tensor out, at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor beta, OptT a,
                  at::Tensor dt_bias, at::Tensor A_log, OptT D, at::Tensor state, at::Tensor state_rows, int64_t off,
                  at::Tensor qsl, at::Tensor seq_lens, int64_t H, int64_t G, int64_t dk, int64_t dv, double q_scale,
-                 double unit_eps) {
+                 double unit_eps, int64_t piece = 1, int64_t npieces = 1, OptT sc_local = OptT(), OptT sc_start = OptT(),
+                 OptT sc_decay = OptT()) {
   const bool bf = is_bf(q);
   const int64_t T = q.size(0), S = seq_lens.numel();
   TORCH_CHECK(G >= 1 && H % G == 0, "heads must divide over the q/k heads (groups)");
@@ -376,14 +377,28 @@ void column_scan(bool delta, at::Tensor out, at::Tensor q, at::Tensor k, at::Ten
   p.dv = static_cast<int>(dv);
   p.q_scale = static_cast<float>(q_scale);
   p.unit_eps = static_cast<float>(unit_eps);
+  p.piece = 1;
+  p.npieces = 1;
+  if (npieces > 1) {  // pieces side by side: scratch [S, npieces, state] twice and [S, npieces, H]
+    TORCH_CHECK(!delta && piece >= 16 && sc_local.has_value() && sc_start.has_value() && sc_decay.has_value(),
+                "a split scan needs its scratch pools");
+    TORCH_CHECK(sc_local->numel() >= S * npieces * H * dk * dv && sc_start->numel() >= S * npieces * H * dk * dv &&
+                sc_decay->numel() >= S * npieces * H, "scratch pools smaller than [S, npieces, state]");
+    p.piece = static_cast<int>(piece);
+    p.npieces = static_cast<int>(npieces);
+    p.sc_local = f32(*sc_local, "sc_local");
+    p.sc_start = f32(*sc_start, "sc_start");
+    p.sc_decay = f32(*sc_decay, "sc_decay");
+  }
   TORCH_CHECK(mxs::launch_column_scan(p, static_cast<int>(S), delta, bf, stream()), "column scan: key / state size beyond 256");
 }
 
 void ssd_scan(at::Tensor out, at::Tensor x, at::Tensor B, at::Tensor C, at::Tensor dt, at::Tensor dt_bias, at::Tensor A_log,
               at::Tensor D, at::Tensor state, at::Tensor state_rows, int64_t off, at::Tensor qsl, at::Tensor seq_lens,
-              int64_t H, int64_t G, int64_t N, int64_t P) {
+              int64_t H, int64_t G, int64_t N, int64_t P, int64_t piece, int64_t npieces, OptT sc_local, OptT sc_start,
+              OptT sc_decay) {
   column_scan(false, out, C, B, x, dt, OptT(), dt_bias, A_log, OptT(D), state, state_rows, off, qsl, seq_lens, H, G, N, P,
-              1.0, 0.0);
+              1.0, 0.0, piece, npieces, sc_local, sc_start, sc_decay);
 }
 
 void delta_scan(at::Tensor out, at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor beta, at::Tensor a, at::Tensor dt_bias,

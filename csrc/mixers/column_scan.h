@@ -26,6 +26,14 @@ struct ScanArgs {
   const int* seq_lens;
   int n_rows, H, G, dk, dv;
   float q_scale, unit_eps;
+  // state space, long chunks cut into pieces that run side by side: mode 0 whole chunk, state from and
+  // to the slot; mode 1 a piece from an empty state, its end state to sc_local and its summed decay
+  // exponents to sc_decay, no outputs; mode 2 a piece from sc_start, outputs, the sequence's last
+  // piece writes the slot
+  int mode, piece, npieces;
+  float* sc_local;   // [S, npieces, H*dv*dk]
+  float* sc_start;   // [S, npieces, H*dv*dk]
+  float* sc_decay;   // [S, npieces, H]
 };
 
 }  // namespace mxs

@@ -7,10 +7,14 @@
 // column's full sum BEFORE the update, is R multiply-adds and four DPP row rotations, with no LDS
 // round trip or barrier inside a token.  Sixteen tokens are staged per barrier pair: the key-side
 // vectors as fp32 in LDS with everything that is per token and head already applied (unit norm,
-// query scale, decays through softplus and exp, write strength), the 16 value columns, and the
-// previous 16 tokens' outputs are written while the next are staged.
+// query scale, decays through softplus and exp, write strength) and the 16 value columns.  The 256
+// threads stage as 16 tokens x 16 runs, the same 16-lane rows as the recurrence, so a unit norm is
+// a DPP row sum too; a stage's global loads are issued before the stage before it is walked, and
+// the previous 16 tokens' outputs are written while the next are staged.
 // A token's sums run in an order fixed by the sizes alone, so cutting a prompt differently gives the
 // same bits.  State, decays, gates and every product are fp32; the operands come as bf16 or fp32.
+#include <algorithm>
+
 #include "mix_common.h"
 #include "column_scan.h"
 
@@ -30,144 +34,311 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
-template <typename T, int R, bool DELTA>
-__global__ void __launch_bounds__(256) column_scan_kernel(const ScanArgs p) {
-  constexpr int DK = 16 * R;  // padded key size
-  __shared__ float sk[kST][DK];
-  __shared__ float sq[kST][DK];
-  __shared__ float sg[DELTA ? kST : 1][DELTA ? DK : 1];
-  __shared__ float sv[kST][kCols];
-  __shared__ float so[kST][kCols];
-  __shared__ float sb[kST], sa[kST];
-  const int s = blockIdx.x, hd = blockIdx.y, c0 = blockIdx.z * kCols;
-  const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
-  const int rp = lane & 15, cl = wid * 4 + (lane >> 4);  // row part; column inside the workgroup
-  const int H = p.H, dk = p.dk, dv = p.dv;
-  const int row0 = p.qsl[s];
-  if (row0 < 0 || row0 >= p.n_rows) return;
-  const int qlen = min(p.qsl[s + 1], p.n_rows) - row0;  // never past the step's rows, whatever the metadata says
-  if (qlen <= 0) return;
-  const bool fresh = p.seq_lens[s] - qlen <= 0;
-  const int col = c0 + cl;
-  const bool col_ok = col < dv;
-  const int kh = hd / (H / p.G);  // the head's q/k head (delta) or B/C group (ssd)
-  float* Sg = p.state + static_cast<long>(p.state_rows[s]) * p.state_stride + p.off +
-              (static_cast<long>(hd) * dv + (col_ok ? col : 0)) * dk + rp * R;
-  float S[R];
+// R consecutive elements as fp32; `vec`: the run is aligned to its own size (16 bytes at most)
+template <int R> __device__ __forceinline__ void load_run(const bf16_t* p, float* o, bool vec) {
+  if (vec) {
+    if constexpr (R >= 8) {
 #pragma unroll
-  for (int i = 0; i < R; ++i) S[i] = (!fresh && col_ok && rp * R + i < dk) ? Sg[i] : 0.f;
+      for (int c = 0; c < R / 8; ++c) {
+        const uint4 a = *reinterpret_cast<const uint4*>(p + 8 * c);
+        o[8 * c] = bf2f_lo(a.x); o[8 * c + 1] = bf2f_hi(a.x); o[8 * c + 2] = bf2f_lo(a.y); o[8 * c + 3] = bf2f_hi(a.y);
+        o[8 * c + 4] = bf2f_lo(a.z); o[8 * c + 5] = bf2f_hi(a.z); o[8 * c + 6] = bf2f_lo(a.w); o[8 * c + 7] = bf2f_hi(a.w);
+      }
+    } else if constexpr (R == 4) {
+      const uint2 a = *reinterpret_cast<const uint2*>(p);
+      o[0] = bf2f_lo(a.x); o[1] = bf2f_hi(a.x); o[2] = bf2f_lo(a.y); o[3] = bf2f_hi(a.y);
+    } else {
+      const uint32_t a = *reinterpret_cast<const uint32_t*>(p);
+      o[0] = bf2f_lo(a); o[1] = bf2f_hi(a);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < R; ++i) o[i] = bf2f(p[i]);
+  }
+}
+template <int R> __device__ __forceinline__ void load_run(const float* p, float* o, bool vec) {
+  if (vec) {
+    if constexpr (R >= 4) {
+#pragma unroll
+      for (int c = 0; c < R / 4; ++c) {
+        const float4 a = *reinterpret_cast<const float4*>(p + 4 * c);
+        o[4 * c] = a.x; o[4 * c + 1] = a.y; o[4 * c + 2] = a.z; o[4 * c + 3] = a.w;
+      }
+    } else {
+      const float2 a = *reinterpret_cast<const float2*>(p);
+      o[0] = a.x; o[1] = a.y;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < R; ++i) o[i] = p[i];
+  }
+}
+template <int R> __device__ __forceinline__ void store_run(float* p, const float* o, bool vec) {
+  if (vec) {
+    if constexpr (R >= 4) {
+#pragma unroll
+      for (int c = 0; c < R / 4; ++c) *reinterpret_cast<float4*>(p + 4 * c) = make_float4(o[4 * c], o[4 * c + 1], o[4 * c + 2], o[4 * c + 3]);
+    } else {
+      *reinterpret_cast<float2*>(p) = make_float2(o[0], o[1]);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < R; ++i) p[i] = o[i];
+  }
+}
+
+// What one thread brings in for a stage: its run of R key-side elements of the token it stages (the
+// token tid / 16; the run is the one whose rows it owns in the recurrence), one value element and the
+// token's scalar.  The loads of a stage are issued before the 16 tokens of the stage before it are
+// walked, so their latency hides behind that walk.
+template <int R, bool DELTA> struct StageRegs {
+  float k[R], q[R], a[DELTA ? R : 1], v, b;
+};
+
+template <typename T, int R, bool DELTA>
+__device__ __forceinline__ void load_stage(StageRegs<R, DELTA>& r, const ScanArgs& p, long row, bool ok, int kh, int hd,
+                                           int rp, int vcol, int flags) {
   const T* qp = static_cast<const T*>(p.q);
   const T* kp = static_cast<const T*>(p.k);
   const T* vp = static_cast<const T*>(p.v);
   const T* bp = static_cast<const T*>(p.beta);
   const T* ap = static_cast<const T*>(p.a);
+  const int d0 = rp * R;
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    r.k[i] = 0.f;
+    r.q[i] = 0.f;
+    if (DELTA) r.a[i] = 0.f;
+  }
+  r.v = 0.f;
+  r.b = 0.f;
+  if (!ok) return;
+  if (d0 + R <= p.dk) {
+    load_run<R>(kp + row * p.k_stride + kh * p.dk + d0, r.k, flags & 1);
+    load_run<R>(qp + row * p.q_stride + kh * p.dk + d0, r.q, flags & 2);
+    if (DELTA) load_run<R>(ap + row * p.a_stride + hd * p.dk + d0, r.a, flags & 4);
+  } else {
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      if (d0 + i < p.dk) {
+        r.k[i] = ldf(kp + row * p.k_stride + kh * p.dk + d0 + i);
+        r.q[i] = ldf(qp + row * p.q_stride + kh * p.dk + d0 + i);
+        if (DELTA) r.a[i] = ldf(ap + row * p.a_stride + hd * p.dk + d0 + i);
+      }
+    }
+  }
+  if (vcol < p.dv) r.v = ldf(vp + row * p.v_stride + hd * p.dv + vcol);
+  r.b = ldf(bp + row * p.beta_stride + hd);
+}
+
+template <typename T, int R, bool DELTA>
+__global__ void __launch_bounds__(256) column_scan_kernel(const ScanArgs p, int flags) {
+  constexpr int DK = 16 * R;  // padded key size
+  __shared__ __attribute__((aligned(16))) float sk[kST][DK];
+  __shared__ __attribute__((aligned(16))) float sq[kST][DK];
+  __shared__ __attribute__((aligned(16))) float sg[DELTA ? kST : 1][DELTA ? DK : 4];
+  __shared__ float sv[kST][kCols];
+  __shared__ float so[kST][kCols];
+  __shared__ float sb[kST], sa[kST];
+  const int mode = p.mode, np = p.npieces;
+  const int s = blockIdx.x / np, pc = blockIdx.x - s * np, hd = blockIdx.y, c0 = blockIdx.z * kCols;
+  const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
+  // recurrence: the thread owns rows rp*R.. of column cl.  staging: run rp of token cl.
+  const int rp = lane & 15, cl = wid * 4 + (lane >> 4);
+  const int H = p.H, dk = p.dk, dv = p.dv;
+  int row0 = p.qsl[s];
+  if (row0 < 0 || row0 >= p.n_rows) return;
+  const int qlen_all = min(p.qsl[s + 1], p.n_rows) - row0;  // never past the step's rows, whatever the metadata says
+  const int tb = mode == 0 ? 0 : pc * p.piece;              // this workgroup's rows of the chunk: [tb, te)
+  const int te = mode == 0 ? qlen_all : min(qlen_all, tb + p.piece);
+  if (te <= tb) return;
+  const int qlen = te - tb;
+  row0 += tb;
+  const bool fresh = mode == 1 || (mode == 0 && p.seq_lens[s] - qlen_all <= 0);
+  const int col = c0 + cl;
+  const bool col_ok = col < dv;
+  const int kh = hd / (H / p.G);  // the head's q/k head (delta rule) or B/C group (state space)
+  const long in_head = (static_cast<long>(hd) * dv + (col_ok ? col : 0)) * dk + rp * R;
+  const long sc_at = (static_cast<long>(s) * np + pc) * (static_cast<long>(H) * dv * dk);
+  float* slot = p.state + static_cast<long>(p.state_rows[s]) * p.state_stride + p.off;
+  const float* Sin = (mode == 2 ? p.sc_start + sc_at : slot) + in_head;
+  float* Sg = (mode == 1 ? p.sc_local + sc_at : slot) + in_head;
+  const bool write_state = mode != 2 || te == qlen_all;
+  const bool run_in = rp * R + R <= dk;
+  float S[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) S[i] = 0.f;
+  if (!fresh && col_ok) {
+    if (run_in) {
+      load_run<R>(Sin, S, flags & 8);
+    } else {
+#pragma unroll
+      for (int i = 0; i < R; ++i)
+        if (rp * R + i < dk) S[i] = Sin[i];
+    }
+  }
+  float dsum = 0.f;  // mode 1: this thread's share of the piece's summed decay exponents
   const float eA = expf(p.A_log[hd]);
   const float Dh = DELTA ? 0.f : p.D[hd];
+  float bias[DELTA ? R : 1];
+  if (DELTA) {
+#pragma unroll
+    for (int i = 0; i < R; ++i) bias[i] = rp * R + i < dk ? p.dt_bias[hd * dk + rp * R + i] : 0.f;
+  } else {
+    bias[0] = p.dt_bias[hd];
+  }
   const int HV = H * dv;
+  StageRegs<R, DELTA> rg;
+  load_stage<T, R, DELTA>(rg, p, row0 + cl, cl < qlen, kh, hd, rp, c0 + rp, flags);
   int prev_t0 = -1, prev_nt = 0;
   for (int t0 = 0; t0 < qlen; t0 += kST) {
     const int nt = min(kST, qlen - t0);
     __syncthreads();  // the previous stage's reads of the staged vectors and writes of so are done
-    if (prev_t0 >= 0) {
-      const int tt = tid >> 4, jj = tid & 15;
-      if (tt < prev_nt && c0 + jj < dv) p.out[static_cast<long>(row0 + prev_t0 + tt) * HV + hd * dv + c0 + jj] = so[tt][jj];
-    }
-    // key-side vectors: wave w stages tokens w, w+4, ...
-    for (int tt = wid; tt < nt; tt += 4) {
-      const long row = row0 + t0 + tt;
-      if (DELTA) {
-        float kq[2][(DK + 63) / 64];
-        float ssk = 0.f, ssq = 0.f;
+    if (mode != 1 && prev_t0 >= 0 && cl < prev_nt && c0 + rp < dv)
+      p.out[static_cast<long>(row0 + prev_t0 + cl) * HV + hd * dv + c0 + rp] = so[cl][rp];
+    // this stage's registers -> LDS, with everything that is per token and head applied
+    if (DELTA) {
+      float ssk = 0.f, ssq = 0.f;
 #pragma unroll
-        for (int c = 0; c < (DK + 63) / 64; ++c) {
-          const int d = lane + 64 * c;
-          const float kv = d < dk ? ldf(kp + row * p.k_stride + kh * dk + d) : 0.f;
-          const float qv = d < dk ? ldf(qp + row * p.q_stride + kh * dk + d) : 0.f;
-          kq[0][c] = kv;
-          kq[1][c] = qv;
-          ssk += kv * kv;
-          ssq += qv * qv;
-        }
-        const float ik = rsqrtf(wave_sum(ssk) + p.unit_eps), iq = rsqrtf(wave_sum(ssq) + p.unit_eps) * p.q_scale;
+      for (int i = 0; i < R; ++i) {
+        ssk += rg.k[i] * rg.k[i];
+        ssq += rg.q[i] * rg.q[i];
+      }
+      const float ik = rsqrtf(row16_sum(ssk) + p.unit_eps), iq = rsqrtf(row16_sum(ssq) + p.unit_eps) * p.q_scale;
 #pragma unroll
-        for (int c = 0; c < (DK + 63) / 64; ++c) {
-          const int d = lane + 64 * c;
-          if (d < DK) {
-            sk[tt][d] = kq[0][c] * ik;
-            sq[tt][d] = kq[1][c] * iq;
-            sg[tt][d] = d < dk ? expf(-eA * softplus_cs(ldf(ap + row * p.a_stride + hd * dk + d) + p.dt_bias[hd * dk + d])) : 0.f;
-          }
-        }
-        if (lane == 0) sb[tt] = sigmoid_f(ldf(bp + row * p.beta_stride + hd));
-      } else {
-        for (int d = lane; d < DK; d += 64) {
-          sk[tt][d] = d < dk ? ldf(kp + row * p.k_stride + kh * dk + d) : 0.f;
-          sq[tt][d] = d < dk ? ldf(qp + row * p.q_stride + kh * dk + d) : 0.f;
-        }
-        if (lane == 0) {
-          const float dt = softplus_cs(ldf(bp + row * p.beta_stride + hd) + p.dt_bias[hd]);
-          sb[tt] = dt;
-          sa[tt] = expf(-eA * dt);
-        }
+      for (int i = 0; i < R; ++i) {
+        sk[cl][rp * R + i] = rg.k[i] * ik;
+        sq[cl][rp * R + i] = rg.q[i] * iq;
+        sg[cl][rp * R + i] = rp * R + i < dk ? expf(-eA * softplus_cs(rg.a[i] + bias[i])) : 0.f;
+      }
+      if (rp == 0) sb[cl] = sigmoid_f(rg.b);
+    } else {
+#pragma unroll
+      for (int i = 0; i < R; ++i) {
+        sk[cl][rp * R + i] = rg.k[i];
+        sq[cl][rp * R + i] = rg.q[i];
+      }
+      if (rp == 0) {
+        const float dt = softplus_cs(rg.b + bias[0]);
+        sb[cl] = dt;
+        sa[cl] = expf(-eA * dt);
+        if (cl < nt) dsum += eA * dt;
       }
     }
-    {
-      const int tt = tid >> 4, jj = tid & 15;
-      sv[tt][jj] = (tt < nt && c0 + jj < dv) ? ldf(vp + static_cast<long>(row0 + t0 + tt) * p.v_stride + hd * dv + c0 + jj) : 0.f;
-    }
+    sv[cl][rp] = rg.v;
     __syncthreads();
-    for (int tt = 0; tt < nt; ++tt) {
+    if (t0 + kST < qlen)  // the next stage's loads fly while this stage's tokens are walked
+      load_stage<T, R, DELTA>(rg, p, row0 + t0 + kST + cl, t0 + kST + cl < qlen, kh, hd, rp, c0 + rp, flags);
+    auto token = [&](int tt) {
       const float vj = sv[tt][cl];
       const float* kr = &sk[tt][rp * R];
       const float* qr = &sq[tt][rp * R];
       float o;
       if (DELTA) {
         const float* gr = &sg[tt][rp * R];
-        float part = 0.f;
+        float p0 = 0.f, p1 = 0.f;
 #pragma unroll
-        for (int i = 0; i < R; ++i) {
+        for (int i = 0; i < R; i += 2) {
           S[i] *= gr[i];
-          part += S[i] * kr[i];
+          S[i + 1] *= gr[i + 1];
+          p0 += S[i] * kr[i];
+          p1 += S[i + 1] * kr[i + 1];
         }
-        const float u = sb[tt] * (vj - row16_sum(part));
-        part = 0.f;
+        const float u = sb[tt] * (vj - row16_sum(p0 + p1));
+        p0 = 0.f;
+        p1 = 0.f;
 #pragma unroll
-        for (int i = 0; i < R; ++i) {
+        for (int i = 0; i < R; i += 2) {
           S[i] += kr[i] * u;
-          part += S[i] * qr[i];
+          S[i + 1] += kr[i + 1] * u;
+          p0 += S[i] * qr[i];
+          p1 += S[i + 1] * qr[i + 1];
         }
-        o = row16_sum(part);
+        o = row16_sum(p0 + p1);
       } else {
         const float a = sa[tt], xb = sb[tt] * vj;
-        float part = 0.f;
+        float p0 = 0.f, p1 = 0.f;
 #pragma unroll
-        for (int i = 0; i < R; ++i) {
+        for (int i = 0; i < R; i += 2) {
           S[i] = a * S[i] + xb * kr[i];
-          part += S[i] * qr[i];
+          S[i + 1] = a * S[i + 1] + xb * kr[i + 1];
+          p0 += S[i] * qr[i];
+          p1 += S[i + 1] * qr[i + 1];
         }
-        o = row16_sum(part) + Dh * vj;
+        o = row16_sum(p0 + p1) + Dh * vj;
       }
       if (rp == 0) so[tt][cl] = o;
+    };
+    if (nt == kST) {
+#pragma unroll 4
+      for (int tt = 0; tt < kST; ++tt) token(tt);
+    } else {
+      for (int tt = 0; tt < nt; ++tt) token(tt);
     }
     prev_t0 = t0;
     prev_nt = nt;
   }
   __syncthreads();
-  {
-    const int tt = tid >> 4, jj = tid & 15;
-    if (tt < prev_nt && c0 + jj < dv) p.out[static_cast<long>(row0 + prev_t0 + tt) * HV + hd * dv + c0 + jj] = so[tt][jj];
+  if (mode != 1 && cl < prev_nt && c0 + rp < dv)
+    p.out[static_cast<long>(row0 + prev_t0 + cl) * HV + hd * dv + c0 + rp] = so[cl][rp];
+  if (mode == 1 && blockIdx.z == 0) {  // the piece's decay: exp(-sum) carries a state across it
+    if (rp == 0) sa[cl] = dsum;
+    __syncthreads();
+    if (tid == 0) {
+      float t = 0.f;
+      for (int i = 0; i < kST; ++i) t += sa[i];
+      p.sc_decay[(static_cast<long>(s) * np + pc) * H + hd] = t;
+    }
   }
-  if (col_ok) {
+  if (col_ok && write_state) {
+    if (run_in) {
+      store_run<R>(Sg, S, flags & 8);
+    } else {
 #pragma unroll
-    for (int i = 0; i < R; ++i)
-      if (rp * R + i < dk) Sg[i] = S[i];
+      for (int i = 0; i < R; ++i)
+        if (rp * R + i < dk) Sg[i] = S[i];
+    }
+  }
+}
+
+// Chains the pieces of a split state-space scan: sc_start[s][p] = the state at the start of piece p, from
+// the slot (or zero for a sequence's first tokens), the pieces' end states from an empty state and
+// their decays.  One thread per state element, pieces walked in order.
+__global__ void __launch_bounds__(256) column_chain_kernel(const ScanArgs p) {
+  const int s = blockIdx.x, hd = blockIdx.y;
+  const long per_head = static_cast<long>(p.dv) * p.dk;
+  const long e = static_cast<long>(blockIdx.z) * 256 + threadIdx.x;
+  if (e >= per_head) return;
+  const int row0 = p.qsl[s];
+  if (row0 < 0 || row0 >= p.n_rows) return;
+  const int qlen = min(p.qsl[s + 1], p.n_rows) - row0;
+  if (qlen <= 0) return;
+  const int np = min((qlen + p.piece - 1) / p.piece, p.npieces);
+  const long at = hd * per_head + e, all = static_cast<long>(p.H) * per_head;
+  const float* slot = p.state + static_cast<long>(p.state_rows[s]) * p.state_stride + p.off;
+  float cur = p.seq_lens[s] - qlen <= 0 ? 0.f : slot[at];
+  for (int pc = 0; pc < np; ++pc) {
+    const long sc = (static_cast<long>(s) * p.npieces + pc) * all + at;
+    p.sc_start[sc] = cur;
+    if (pc == np - 1) break;
+    cur = expf(-p.sc_decay[(static_cast<long>(s) * p.npieces + pc) * p.H + hd]) * cur + p.sc_local[sc];
   }
 }
 
 template <typename T, bool DELTA>
 static bool launch_cs(const ScanArgs& a, int S, hipStream_t st) {
-  const dim3 grid(S, a.H, (a.dv + kCols - 1) / kCols), block(256);
-#define MIX_CS(R) hipLaunchKernelGGL((column_scan_kernel<T, R, DELTA>), grid, block, 0, st, a)
+  const dim3 grid(S * a.npieces, a.H, (a.dv + kCols - 1) / kCols), block(256);
+  const int R = a.dk <= 32 ? 2 : a.dk <= 64 ? 4 : a.dk <= 128 ? 8 : 16;
+  // which operands' runs of R elements are aligned to their size (16 bytes at most): 1 k, 2 q, 4 a, 8 state
+  const size_t es = sizeof(T), al = std::min<size_t>(16, R * es), sal = std::min<size_t>(16, R * 4);
+  auto ok = [&](const void* ptr, long stride) {
+    return ptr != nullptr && reinterpret_cast<uintptr_t>(ptr) % al == 0 && (stride * es) % al == 0 && (a.dk * es) % al == 0;
+  };
+  int flags = (ok(a.k, a.k_stride) ? 1 : 0) | (ok(a.q, a.q_stride) ? 2 : 0) | (DELTA && ok(a.a, a.a_stride) ? 4 : 0);
+  if (reinterpret_cast<uintptr_t>(a.state) % sal == 0 && (a.state_stride * 4) % sal == 0 && (a.off * 4) % sal == 0 &&
+      (a.dk * 4) % sal == 0)
+    flags |= 8;
+#define MIX_CS(R) hipLaunchKernelGGL((column_scan_kernel<T, R, DELTA>), grid, block, 0, st, a, flags)
   if (a.dk <= 32) MIX_CS(2);
   else if (a.dk <= 64) MIX_CS(4);
   else if (a.dk <= 128) MIX_CS(8);
@@ -178,10 +349,27 @@ static bool launch_cs(const ScanArgs& a, int S, hipStream_t st) {
   return true;
 }
 
-bool launch_column_scan(const ScanArgs& a, int S, bool delta, bool bf, hipStream_t st) {
-  if (S == 0 || a.n_rows == 0) return true;
+static bool launch_pass(const ScanArgs& a, int S, bool delta, bool bf, hipStream_t st) {
   if (bf) return delta ? launch_cs<bf16_t, true>(a, S, st) : launch_cs<bf16_t, false>(a, S, st);
   return delta ? launch_cs<float, true>(a, S, st) : launch_cs<float, false>(a, S, st);
+}
+
+bool launch_column_scan(const ScanArgs& a0, int S, bool delta, bool bf, hipStream_t st) {
+  if (S == 0 || a0.n_rows == 0) return true;
+  ScanArgs a = a0;
+  if (delta || a.npieces <= 1) {  // the delta rule's step is no diagonal map: its chunks are walked whole
+    a.mode = 0;
+    a.piece = 1;
+    a.npieces = 1;
+    return launch_pass(a, S, delta, bf, st);
+  }
+  a.mode = 1;
+  if (!launch_pass(a, S, false, bf, st)) return false;
+  const long per_head = static_cast<long>(a.dv) * a.dk;
+  hipLaunchKernelGGL(column_chain_kernel, dim3(S, a.H, static_cast<unsigned>((per_head + 255) / 256)), dim3(256), 0, st, a);
+  MXS_CHECK_LAUNCH();
+  a.mode = 2;
+  return launch_pass(a, S, false, bf, st);
 }
 
 }  // namespace mxs

@@ -120,32 +120,79 @@ __global__ void __launch_bounds__(64) rope_rows_kernel(T* __restrict__ out, long
   }
 }
 
-// y[t, c] = act(bias[c] + sum_j w[c, j] x[t - (taps-1) + j, c]); inputs before the chunk come from the
-// sequence's state rows [taps-1, C] (oldest first), zeros for a sequence's first tokens.
-template <typename T>
+// y[t, c] = act(bias[c] + sum_j w[j, c] x[t - (taps-1) + j, c]), w tap-major [taps, C]; inputs before the
+// chunk come from the sequence's state rows [taps-1, C] (oldest first), zeros for a sequence's first
+// tokens.  A thread takes V consecutive channels: V = 16 bytes' worth when rows, weights and channel
+// count allow whole 16-byte pieces, else 1.
+template <typename T> struct Piece;
+template <> struct Piece<bf16_t> { static constexpr int N = 8; };
+template <> struct Piece<float> { static constexpr int N = 4; };
+__device__ __forceinline__ void load_piece(const bf16_t* p, float* o) {
+  const uint4 a = *reinterpret_cast<const uint4*>(p);
+  o[0] = bf2f_lo(a.x); o[1] = bf2f_hi(a.x); o[2] = bf2f_lo(a.y); o[3] = bf2f_hi(a.y);
+  o[4] = bf2f_lo(a.z); o[5] = bf2f_hi(a.z); o[6] = bf2f_lo(a.w); o[7] = bf2f_hi(a.w);
+}
+__device__ __forceinline__ void load_piece(const float* p, float* o) {
+  const float4 a = *reinterpret_cast<const float4*>(p);
+  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+}
+__device__ __forceinline__ void store_piece(bf16_t* p, const float* o) {
+  uint4 a;
+  a.x = pack2(o[0], o[1]); a.y = pack2(o[2], o[3]); a.z = pack2(o[4], o[5]); a.w = pack2(o[6], o[7]);
+  *reinterpret_cast<uint4*>(p) = a;
+}
+__device__ __forceinline__ void store_piece(float* p, const float* o) {
+  *reinterpret_cast<float4*>(p) = make_float4(o[0], o[1], o[2], o[3]);
+}
+
+template <typename T, bool WIDE>
 __global__ void __launch_bounds__(256) causal_conv_kernel(T* __restrict__ out, const T* __restrict__ x, long x_stride,
                                                           const T* __restrict__ w, const T* __restrict__ bias,
                                                           const float* __restrict__ state, long state_stride,
                                                           const int* __restrict__ state_rows, long off,
                                                           const int* __restrict__ qsl, const int* __restrict__ seq_lens,
                                                           int S, int C, int taps, int silu) {
+  constexpr int V = WIDE ? Piece<T>::N : 1;
   const int t = blockIdx.x;
-  const int c = blockIdx.y * 256 + threadIdx.x;
+  const int c = (blockIdx.y * 256 + threadIdx.x) * V;
   if (c >= C) return;
   const int s = seq_of_row(qsl, S, t);
   const int row0 = qsl[s], qlen = qsl[s + 1] - row0;
   const int i = t - row0;
   const bool fresh = seq_lens[s] - qlen <= 0;
   const float* st = state + static_cast<long>(state_rows[s]) * state_stride + off;
-  float acc = bias ? ldf(bias + c) : 0.f;
+  float acc[V], xv[V], wv[V];
+  if constexpr (WIDE) {
+    if (bias) load_piece(bias + c, acc);
+    else for (int e = 0; e < V; ++e) acc[e] = 0.f;
+  } else {
+    acc[0] = bias ? ldf(bias + c) : 0.f;
+  }
   for (int j = 0; j < taps; ++j) {
     const int src = i - (taps - 1 - j);
-    float xv = 0.f;
-    if (src >= 0) xv = ldf(x + static_cast<long>(row0 + src) * x_stride + c);
-    else if (!fresh) xv = st[static_cast<long>(taps - 1 + src) * C + c];
-    acc += ldf(w + static_cast<long>(c) * taps + j) * xv;
+    if (src < 0 && fresh) continue;
+    if constexpr (WIDE) {
+      if (src >= 0) {
+        load_piece(x + static_cast<long>(row0 + src) * x_stride + c, xv);
+      } else {
+        const float* sp = st + static_cast<long>(taps - 1 + src) * C + c;
+#pragma unroll
+        for (int e = 0; e < V; e += 4) load_piece(sp + e, xv + e);
+      }
+      load_piece(w + static_cast<long>(j) * C + c, wv);
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] += wv[e] * xv[e];
+    } else {
+      xv[0] = src >= 0 ? ldf(x + static_cast<long>(row0 + src) * x_stride + c) : st[static_cast<long>(taps - 1 + src) * C + c];
+      acc[0] += ldf(w + static_cast<long>(j) * C + c) * xv[0];
+    }
   }
-  stf(out + static_cast<long>(t) * C + c, silu ? silu_f(acc) : acc);
+  if (silu) {
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc[e] = silu_f(acc[e]);
+  }
+  if constexpr (WIDE) store_piece(out + static_cast<long>(t) * C + c, acc);
+  else stf(out + static_cast<long>(t) * C + c, acc[0]);
 }
 
 // The state after the step: the last taps-1 inputs of (old state ++ chunk).  Row r of the new state
@@ -266,9 +313,21 @@ void launch_causal_conv(void* out, const void* x, long x_stride, const void* w, 
                         int rows, int C, int taps, int silu, bool bf, hipStream_t st) {
   if (rows == 0 || S == 0) return;
   const int cb = (C + 255) / 256;
-  MIX_DISPATCH(bf, hipLaunchKernelGGL(causal_conv_kernel<T>, dim3(rows, cb), dim3(256), 0, st, (T*)out, (const T*)x,
-                                      x_stride, (const T*)w, (const T*)bias, state, state_stride, state_rows, off, qsl,
-                                      seq_lens, S, C, taps, silu));
+  // whole 16-byte pieces everywhere: rows, weights, bias, output, and the fp32 state rows
+  const int v = bf ? 8 : 4;
+  auto al = [](const void* ptr) { return reinterpret_cast<uintptr_t>(ptr) % 16 == 0; };
+  const bool wide = C % v == 0 && x_stride % v == 0 && al(x) && al(w) && al(out) && (bias == nullptr || al(bias)) &&
+                    al(state) && state_stride % 4 == 0 && off % 4 == 0;
+  if (wide) {
+    const int cw = (C / v + 255) / 256;
+    MIX_DISPATCH(bf, hipLaunchKernelGGL((causal_conv_kernel<T, true>), dim3(rows, cw), dim3(256), 0, st, (T*)out,
+                                        (const T*)x, x_stride, (const T*)w, (const T*)bias, state, state_stride,
+                                        state_rows, off, qsl, seq_lens, S, C, taps, silu));
+  } else {
+    MIX_DISPATCH(bf, hipLaunchKernelGGL((causal_conv_kernel<T, false>), dim3(rows, cb), dim3(256), 0, st, (T*)out,
+                                        (const T*)x, x_stride, (const T*)w, (const T*)bias, state, state_stride,
+                                        state_rows, off, qsl, seq_lens, S, C, taps, silu));
+  }
   MXS_CHECK_LAUNCH();
   if (taps > 1) {
     MIX_DISPATCH(bf, hipLaunchKernelGGL(conv_state_kernel<T>, dim3(S, cb), dim3(256), 0, st, (const T*)x, x_stride, state,

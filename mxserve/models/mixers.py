@@ -320,6 +320,7 @@ class Mamba2(Mixer):
     def finish_weights(self, w: dict) -> None:
         for n in ("dt_bias", "A_log", "D"):
             _fp32(w, self.p + n)
+        w[self.p + "conv"] = w[self.p + "conv"].t().contiguous()  # tap-major for the kernel
 
     def mix(self, parts: list, h: torch.Tensor, w: dict, ctx: StepContext, koff: int, voff: int, soff: int,
             out: Optional[torch.Tensor] = None, out_scale: float = 1.0) -> torch.Tensor:
@@ -331,7 +332,7 @@ class Mamba2(Mixer):
                                md.query_start_loc, md.seq_lens, silu=True)
         o = seqmix.ssd_scan(c[:, :I], c[:, I:I + GN], c[:, I + GN:], dt, w[p + "dt_bias"], w[p + "A_log"], w[p + "D"],
                             ctx.state, md.state_rows, soff, md.query_start_loc, md.seq_lens, self.heads, self.G,
-                            self.N, self.P)
+                            self.N, self.P, max_query_len=md.max_query_len)
         return seqmix.gated_norm(o, z, w[p + "norm"], ctx.eps, self.norm_groups, "silu", True, h.dtype, out_scale, out)
 
     def forward(self, parts: list, h: torch.Tensor, w: dict, ctx: StepContext, koff: int, voff: int, soff: int):
@@ -380,7 +381,8 @@ class GatedDeltaRule(Mixer):
 
     def finish_weights(self, w: dict) -> None:
         p = self.p
-        w[p + "_conv"] = torch.cat([w.pop(p + "q.conv"), w.pop(p + "k.conv"), w.pop(p + "v.conv")]).contiguous()
+        # one filter over q, k, v's channels, tap-major for the kernel
+        w[p + "_conv"] = torch.cat([w.pop(p + "q.conv"), w.pop(p + "k.conv"), w.pop(p + "v.conv")]).t().contiguous()
         _fp32(w, p + "dt_bias")
         _fp32(w, p + "A_log")
 

@@ -400,12 +400,13 @@ def rope_rows(x: torch.Tensor, positions: torch.Tensor, heads: int, dim: int, fr
 def causal_conv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor,
                 state_rows: torch.Tensor, off: int, qsl: torch.Tensor, seq_lens: torch.Tensor,
                 silu: bool = True) -> torch.Tensor:
-    """Per-channel causal filter over time: y[t, c] = bias[c] + sum_j w[c, j] x[t - (taps-1) + j, c], the
-    last column of w weighing the current token, inputs before a sequence's start being zero; then
-    SiLU.  x [T, C] (row-strided view), w [C, taps].  The sequence's last taps - 1 inputs live in its
-    state slot at `off` as fp32 [taps - 1, C], oldest first, and are replaced by this step's."""
+    """Per-channel causal filter over time: y[t, c] = bias[c] + sum_j w[j, c] x[t - (taps-1) + j, c], the
+    last row of w weighing the current token, inputs before a sequence's start being zero; then
+    SiLU.  x [T, C] (row-strided view), w tap-major [taps, C] (a checkpoint's [C, taps] transposed, so
+    that neighbouring channels' weights are neighbours).  The sequence's last taps - 1 inputs live in
+    its state slot at `off` as fp32 [taps - 1, C], oldest first, and are replaced by this step's."""
     T, C = x.shape
-    taps = w.shape[1]
+    taps = w.shape[0]
     if _gpu(x):
         out = torch.empty(T, C, dtype=x.dtype, device=x.device)
         ext().causal_conv(out, x, w, bias, state, state_rows, int(off), qsl, seq_lens, bool(silu))
@@ -423,7 +424,7 @@ def causal_conv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
         full = torch.cat([prev, x[a:e].float()])
         y = torch.zeros(n, C) if bias is None else bias.float().expand(n, C).clone()
         for j in range(taps):
-            y += wf[:, j] * full[j:j + n]
+            y += wf[j] * full[j:j + n]
         out[a:e] = y
         if taps > 1:
             st.copy_(full[n:])
@@ -433,17 +434,24 @@ def causal_conv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
 # ----------------------------------------------------------------------------- column scans
 def ssd_scan(x: torch.Tensor, B: torch.Tensor, C: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor,
              A_log: torch.Tensor, D: torch.Tensor, state: torch.Tensor, state_rows: torch.Tensor, off: int,
-             qsl: torch.Tensor, seq_lens: torch.Tensor, num_heads: int, groups: int, N: int, P: int) -> torch.Tensor:
+             qsl: torch.Tensor, seq_lens: torch.Tensor, num_heads: int, groups: int, N: int, P: int,
+             max_query_len: int = 0) -> torch.Tensor:
     """Selective state-space recurrence with a scalar decay per head and token (state-space duality):
         d = softplus(dt + dt_bias_h);  S = exp(-exp(A_log_h) d) S + d B_g x_h^T;  y_h = S^T C_g + D_h x_h
     with S [N, P] per head and head h reading group h // (H / G).  x [T, H*P], B, C [T, G*N], dt [T, H]
     (row-strided views of any float dtype); dt_bias, A_log, D fp32 [H].  Returns y fp32 [T, H*P]; the
-    state (fp32, stored [H, P, N]) stays in the sequence's slot."""
+    state (fp32, stored [H, P, N]) stays in the sequence's slot.  max_query_len: the step's longest
+    chunk (host int); the step is a diagonal map of the state, so long chunks are cut into pieces
+    that run side by side (a piece's end state from an empty state, the true state at every piece's
+    start chained from those and the pieces' decays, then the outputs)."""
     T = x.shape[0]
     H = num_heads
     if _gpu(x):
         out = torch.empty(T, H * P, dtype=torch.float32, device=x.device)
-        ext().ssd_scan(out, x, B, C, dt, dt_bias, A_log, D, state, state_rows, int(off), qsl, seq_lens, H, groups, N, P)
+        piece, npieces, loc, start = _scan_split(seq_lens.numel(), T, max_query_len, H * N * P, H, 4 * P, x.device)
+        dec = torch.empty(seq_lens.numel() * npieces * H, dtype=torch.float32, device=x.device) if npieces > 1 else None
+        ext().ssd_scan(out, x, B, C, dt, dt_bias, A_log, D, state, state_rows, int(off), qsl, seq_lens, H, groups, N, P,
+                       piece, npieces, loc, start, dec)
         return out
     out = torch.zeros(T, H, P, dtype=torch.float32)
     xf = x.float().reshape(T, H, P)

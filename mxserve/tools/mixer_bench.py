@@ -1,8 +1,10 @@
-"""Prefill and decode throughput of Voletar beside a Llama-shaped model of equal width, depth and
-feed-forward size (random weights), through the same engine path: forced steps of the scheduler,
-the model runner, paged K/V and state slots, decode through the captured graphs.
+"""Prefill and decode throughput of a layer-list design (Voletar, Tapasun) beside the models closest
+to it at equal width, depth and feed-forward size (random weights), through the same engine path:
+forced steps of the scheduler, the model runner, paged K/V and state slots, decode through the
+captured graphs.  Voletar stands beside a Llama-shaped model; Tapasun beside Voletar and that model.
 
-  python bench.py --mixer-bench [--mixer-sizes 1024,2048] [--mixer-prompt 4096] [--mixer-batch 64]
+  python bench.py --mixer-bench [--mixer-design voletar|tapasun] [--mixer-sizes 1024,2048]
+                  [--mixer-prompt 4096] [--mixer-batch 64]
 
 Prints one JSON line per (size, model): prefill tokens/s of one prompt in one step, decode tokens/s
 of a batch of sequences at that context, and per-kernel times of the mixers against their
@@ -40,7 +42,31 @@ def voletar_shape(width: int, layers: int = 4, window: int = 1024) -> dict:
             "layers": [par if i % 2 == 0 else lig for i in range(layers)]}
 
 
-def register(width: int, layers: int) -> tuple:
+def tapasun_shape(width: int, layers: int = 4) -> dict:
+    """State space, attention, parallel (attention + delta rule), attention on the second layer's pages,
+    with the head sizes of a model of this width and a gated feed-forward of 8/3 width."""
+    hq = width // 64
+    ffn = {"kind": "dense", "ff": (8 * width // 3) // 256 * 256}
+    bands = {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}
+    att = {"heads": hq, "kv_heads": max(hq // 4, 1), "dim": 64, "vdim": 64, "scale": 0.125,
+           "rot": {"dims": 64, "base": 500000.0, "scaling": bands}}
+    ssm = {"type": "mamba2", "mlp": ffn, "mixer": {"heads": width // 32, "vdim": 64, "state": 128,
+                                                  "groups": min(8, width // 32), "conv": 4, "norm_groups": min(8, width // 32)}}
+    gh = max(width // 128, 1)
+    par = {"type": "parallel", "mlp": ffn, "mixer": {
+        "left": {"heads": hq, "kv_heads": max(hq // 8, 1), "dim": 64, "vdim": 64, "scale": 0.125,
+                 "rot": {"dims": 32, "base": 500000.0, "scaling": {"factor": 4.0}}},
+        "right": {"heads": gh, "kv_heads": gh, "dim": 128, "vdim": 128, "conv": 4}, "left_scale": 0.5, "right_scale": 1.0}}
+    kinds = [ssm, {"type": "attention", "mlp": ffn, "mixer": att}, par,
+             {"type": "attention", "mlp": ffn, "mixer": dict(att, kv_from=1)}]
+    return {"architecture": "Tapasun", "width": width, "vocab": 32000, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
+            "layers": [kinds[i % 4] for i in range(layers)]}
+
+
+def register(width: int, layers: int, design: str = "voletar") -> tuple:
+    if design == "tapasun":
+        t = mcfg.tapasun_config(f"tapasun-w{width}", tapasun_shape(width, layers))
+        mcfg.REGISTRY[t.name.lower()] = t
     v = mcfg.voletar_config(f"voletar-w{width}", voletar_shape(width, layers))
     mcfg.REGISTRY[v.name.lower()] = v
     base = mcfg.REGISTRY["small-llama"]
@@ -49,7 +75,7 @@ def register(width: int, layers: int) -> tuple:
                             num_layers=layers, num_heads=width // 64, num_kv_heads=max(width // 256, 1), head_dim=64,
                             vocab_size=32000, tie_word_embeddings=False)
     mcfg.REGISTRY[l.name.lower()] = l
-    return v.name, l.name
+    return (t.name, v.name, l.name) if design == "tapasun" else (v.name, l.name)
 
 
 def _time(fn, reps: int) -> float:
@@ -161,16 +187,97 @@ def kernel_rooflines(width: int, prompt: int, batch: int, context: int) -> list:
     return out
 
 
-def main(sizes: list, prompt: int, batch: int, context: int, layers: int = 4, only: str = "all") -> int:
-    """only: all | voletar | llama | kernels (e.g. one model alone under a profiler)."""
+def tapasun_rooflines(width: int, prompt: int, batch: int, context: int) -> list:
+    """Tapasun's own kernels alone, at the sizes of tapasun_shape(width): time over roofline time.  The
+    like kernels of Voletar (kernel_rooflines) are what they stand beside: its scans for the column
+    scans, its windowed attention for the attention with a sink, its gated norm and cache write for
+    the small kernels."""
+    from ..models.mixers import rotary_frequencies
+    from ..ops import seqmix
+    dev = torch.device("cuda")
+    dt = torch.bfloat16
+    bs, out = 16, []
+    i32 = dict(dtype=torch.int32, device=dev)
+    rnd = lambda *sh: torch.randn(*sh, device=dev).to(dt)  # noqa: E731
+
+    def entry(name, t, flops, peak, bytes_, note):
+        roof = max(flops / peak, bytes_ / PEAK_HBM)
+        out.append({"kernel": name, "width": width, "ms": round(1e3 * t, 4), "roofline_ms": round(1e3 * roof, 4),
+                    "x_roofline": round(t / roof, 1), "counts": note})
+
+    for mode, T, S, ctx in (("prefill", prompt, 1, prompt), ("decode", batch, batch, context)):
+        qsl = torch.arange(0, T + 1, T // S, **i32)
+        seq = torch.full((S,), ctx, **i32)
+        rows = torch.arange(S, **i32)
+        nb = -(-ctx // bs)
+        bt = torch.arange(S * nb, **i32).view(S, nb)
+        pos = torch.cat([torch.arange(ctx - T // S, ctx, device=dev) for _ in range(S)])
+        slots = torch.cat([bt[s_].long().repeat_interleave(bs)[ctx - T // S:ctx] * bs + pos[:T // S] % bs for s_ in range(S)])
+        # attention with a sink, every earlier key visible
+        H, G, dk, dv = width // 64, max(width // 256, 1), 64, 64
+        cache = rnd(S * nb, G * bs * (dk + dv))
+        q, k, v = rnd(T, H * dk), rnd(T, G * dk), rnd(T, G * dv)
+        sink = torch.zeros(H, device=dev)
+        t = _time(lambda: seqmix.window_attention(q, cache, bt, qsl, seq, 0, G * bs * dk, H, G, dk, dv, bs, 0.125, 0, 0,
+                                                  max_query_len=T // S, sink=sink), 5)
+        keys = ctx if mode == "decode" else ctx / 2
+        entry(f"sink_attention/{mode}", t, 2.0 * T * H * keys * (dk + dv), PEAK_BF16,
+              2.0 * (S * ctx * G * (dk + dv) + 2 * T * H * dk), f"{T} rows x {H} heads x ~{int(keys)} keys, bf16 MFMA peak")
+        fr = rotary_frequencies(dk, 500000.0, None).to(dev)
+        nw = torch.ones(dk, device=dev).to(dt)
+        t = _time(lambda: seqmix.rope_qkv_cache(q, k, v, pos, slots, cache, 0, G * bs * dk, H, G, dk, dv, bs, fr, nw, nw,
+                                                1e-5, None), 5)
+        entry(f"rope_qkv_cache/{mode}", t, 0.0, PEAK_F32, 2.0 * T * (2 * H * dk + 2 * G * (dk + dv)),
+              f"{T} rows: q read and written, k and v read and written to the pages")
+        # column scans: fp32 state; 4 (state space) or 7 (delta rule) flops per state element and token
+        for name, Hh, Gg, d1, d2, fl in (("ssd_scan", width // 32, min(8, width // 32), 128, 64, 4.0),
+                                         ("delta_scan", max(width // 128, 1), max(width // 128, 1), 128, 128, 7.0)):
+            n = Hh * d1 * d2
+            state = torch.zeros(S, n, device=dev)
+            qq, kk, vv, bb = rnd(T, Gg * d1), rnd(T, Gg * d1), rnd(T, Hh * d2), rnd(T, Hh)
+            hb = torch.zeros(Hh, device=dev)
+            if name == "ssd_scan":
+                fn = lambda: seqmix.ssd_scan(vv, kk, qq, bb, hb, hb, hb, state, rows, 0, qsl, seq, Hh, Gg, d1, d2,  # noqa: E731
+                                             max_query_len=T // S)
+                extra = 0
+            else:
+                aa = rnd(T, Hh * d1)
+                cb = torch.zeros(Hh * d1, device=dev)
+                fn = lambda: seqmix.delta_scan(qq, kk, vv, bb, aa, cb, hb, state, rows, 0, qsl, seq, Hh, Gg, d1, d2,  # noqa: E731
+                                               d1 ** -0.5)
+                extra = T * Hh * d1
+            t = _time(fn, 5)
+            entry(f"{name}/{mode}", t, fl * T * Hh * d1 * d2, PEAK_F32,
+                  8.0 * S * n + 2.0 * (T * (2 * Gg * d1 + Hh * d2) + extra) + 4.0 * T * Hh * d2,
+                  f"{T} rows x {Hh} heads x {d1}x{d2} state, fp32 peak; state read and written once")
+        # short convolution over the state-space layer's channels, and its gated norm
+        C = 2 * width + 2 * min(8, width // 32) * 128
+        x, wc, bc = rnd(T, C), rnd(4, C), rnd(C)
+        cst = torch.zeros(S, 3 * C, device=dev)
+        t = _time(lambda: seqmix.causal_conv(x, wc, bc, cst, rows, 0, qsl, seq), 5)
+        entry(f"causal_conv/{mode}", t, 0.0, PEAK_F32, 4.0 * T * C + 24.0 * S * C, f"{T} rows x {C} channels, 4 taps; rows read and written once")
+        N = 2 * width
+        o, gate, wn = torch.randn(T, N, device=dev), rnd(T, N), rnd(N)
+        t = _time(lambda: seqmix.gated_norm(o, gate, wn, 1e-5, 8, "silu", True, dt), 5)
+        entry(f"gated_norm/{mode}", t, 0.0, PEAK_F32, 8.0 * T * N, f"{T} rows x {N}: fp32 in, gate in, bf16 out")
+        t = _time(lambda: seqmix.gated_rms_norm(o, gate, wn, 1e-5, 8, dt), 5)
+        entry(f"gated_rms_norm/{mode} (voletar)", t, 0.0, PEAK_F32, 8.0 * T * N, f"{T} rows x {N}: fp32 in, gate in, bf16 out")
+    return out
+
+
+def main(sizes: list, prompt: int, batch: int, context: int, layers: int = 4, only: str = "all",
+         design: str = "voletar") -> int:
+    """only: all | tapasun | voletar | llama | kernels (e.g. one model alone under a profiler)."""
     from .. import ops
     ops.ext()
     for width in sizes:
-        v, l = register(width, layers)
-        for name, key in ((v, "voletar"), (l, "llama")):
-            if only in ("all", key):
+        names = register(width, layers, design)
+        for name in names:
+            if only in ("all", name.split("-")[0]):
                 print(json.dumps(run_model(name, prompt, batch, context)), flush=True)
         if only in ("all", "kernels"):
-            for e in kernel_rooflines(width, prompt, batch, context):
+            rows = (tapasun_rooflines(width, prompt, batch, context) if design == "tapasun" else []) + \
+                kernel_rooflines(width, prompt, batch, context)
+            for e in rows:
                 print(json.dumps(e), flush=True)
     return 0

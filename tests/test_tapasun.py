@@ -149,6 +149,23 @@ def test_state_space_mixer(dev, portions):
 
 
 @pytest.mark.parametrize("dev", DEVS)
+@pytest.mark.parametrize("portions", [[300], [129, 171], [7, 290, 3], [150, 1, 149]])
+def test_state_space_long_chunks(dev, portions):
+    """Chunks long enough that the GPU scan cuts them into pieces that run side by side: a piece's
+    start state is chained from the pieces before it, and from the slot when the chunk is not the
+    sequence's first."""
+    _skip(dev)
+    width, T = 64, 300
+    h = torch.randn(T, width, generator=torch.Generator().manual_seed(4))
+    mc = mamba2(heads=4, vdim=24, state=40, groups=2, conv=3, norm_groups=1)["mixer"]
+    m, w = _mixer_setup("mamba2", mc, width)
+    w["m.A_log"] = w["m.A_log"] - 2.0  # slow decays: what a piece inherits matters to its end
+    wn = {k: v.double().numpy() for k, v in w.items()}
+    want = _oracle_steps(to.Mamba2(mc, wn, "m.", EPS), h.double().numpy())
+    _check(_run_mixers([m], [w], h, dev, portions)[0], want, 1e-4)
+
+
+@pytest.mark.parametrize("dev", DEVS)
 @pytest.mark.parametrize("portions", PORTIONS)
 def test_rotary_attention_mixer_and_shared_pages(dev, portions):
     """An attention layer with keys of its own and a second one that reads the first one's pages with
