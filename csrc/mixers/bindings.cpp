@@ -338,7 +338,7 @@ void column_scan(bool delta, at::Tensor out, at::Tensor q, at::Tensor k, at::Ten
                  at::Tensor dt_bias, at::Tensor A_log, OptT D, at::Tensor state, at::Tensor state_rows, int64_t off,
                  at::Tensor qsl, at::Tensor seq_lens, int64_t H, int64_t G, int64_t dk, int64_t dv, double q_scale,
                  double unit_eps, int64_t piece = 1, int64_t npieces = 1, OptT sc_local = OptT(), OptT sc_start = OptT(),
-                 OptT sc_decay = OptT()) {
+                 OptT sc_decay = OptT(), int64_t mode = 0) {
   const bool bf = is_bf(q);
   const int64_t T = q.size(0), S = seq_lens.numel();
   TORCH_CHECK(G >= 1 && H % G == 0, "heads must divide over the q/k heads (groups)");
@@ -380,15 +380,18 @@ void column_scan(bool delta, at::Tensor out, at::Tensor q, at::Tensor k, at::Ten
   p.piece = 1;
   p.npieces = 1;
   if (npieces > 1) {  // pieces side by side: scratch [S, npieces, state] twice and [S, npieces, H]
-    TORCH_CHECK(!delta && piece >= 16 && sc_local.has_value() && sc_start.has_value() && sc_decay.has_value(),
+    TORCH_CHECK(piece >= 16 && sc_local.has_value() && sc_start.has_value() && (delta || sc_decay.has_value()),
                 "a split scan needs its scratch pools");
-    TORCH_CHECK(sc_local->numel() >= S * npieces * H * dk * dv && sc_start->numel() >= S * npieces * H * dk * dv &&
-                sc_decay->numel() >= S * npieces * H, "scratch pools smaller than [S, npieces, state]");
+    TORCH_CHECK(sc_local->numel() >= S * npieces * H * dk * (delta ? dv + dk : dv) &&
+                sc_start->numel() >= S * npieces * H * dk * dv && (delta || sc_decay->numel() >= S * npieces * H),
+                "scratch pools smaller than [S, npieces, state]");
+    TORCH_CHECK(!delta || mode == 1 || mode == 2, "a split delta-rule scan is launched pass by pass");
     p.piece = static_cast<int>(piece);
     p.npieces = static_cast<int>(npieces);
+    p.mode = static_cast<int>(mode);
     p.sc_local = f32(*sc_local, "sc_local");
     p.sc_start = f32(*sc_start, "sc_start");
-    p.sc_decay = f32(*sc_decay, "sc_decay");
+    p.sc_decay = delta ? nullptr : f32(*sc_decay, "sc_decay");
   }
   TORCH_CHECK(mxs::launch_column_scan(p, static_cast<int>(S), delta, bf, stream()), "column scan: key / state size beyond 256");
 }
@@ -403,9 +406,10 @@ void ssd_scan(at::Tensor out, at::Tensor x, at::Tensor B, at::Tensor C, at::Tens
 
 void delta_scan(at::Tensor out, at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor beta, at::Tensor a, at::Tensor dt_bias,
                 at::Tensor A_log, at::Tensor state, at::Tensor state_rows, int64_t off, at::Tensor qsl, at::Tensor seq_lens,
-                int64_t H, int64_t G, int64_t dk, int64_t dv, double q_scale, double unit_eps) {
+                int64_t H, int64_t G, int64_t dk, int64_t dv, double q_scale, double unit_eps, int64_t mode, int64_t piece,
+                int64_t npieces, OptT sc_local, OptT sc_start) {
   column_scan(true, out, q, k, v, beta, OptT(a), dt_bias, A_log, OptT(), state, state_rows, off, qsl, seq_lens, H, G, dk, dv,
-              q_scale, unit_eps);
+              q_scale, unit_eps, piece, npieces, sc_local, sc_start, OptT(), mode);
 }
 
 }  // namespace

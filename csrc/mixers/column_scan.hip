@@ -11,6 +11,11 @@
 // threads stage as 16 tokens x 16 runs, the same 16-lane rows as the recurrence, so a unit norm is
 // a DPP row sum too; a stage's global loads are issued before the stage before it is walked, and
 // the previous 16 tokens' outputs are written while the next are staged.
+// Long chunks are cut into pieces that run side by side: pass 1 runs every piece from an empty state
+// and keeps its end state, and what carries a state across the piece (state space: the summed decay
+// exponents; delta rule: the piece's dk x dk transition matrix, from dk more columns started as the
+// identity); the states at the pieces' starts are chained from those; pass 2 runs every piece again
+// from its true start and writes the outputs.
 // A token's sums run in an order fixed by the sizes alone, so cutting a prompt differently gives the
 // same bits.  State, decays, gates and every product are fp32; the operands come as bf16 or fp32.
 #include <algorithm>
@@ -155,14 +160,20 @@ __global__ void __launch_bounds__(256) column_scan_kernel(const ScanArgs p, int 
   const int qlen = te - tb;
   row0 += tb;
   const bool fresh = mode == 1 || (mode == 0 && p.seq_lens[s] - qlen_all <= 0);
+  // delta rule, pass 1: dk more columns, started as the identity and fed no values, end as the piece's
+  // transition matrix (the state at the piece's end is that matrix times the state at its start, plus
+  // the end state from an empty start)
+  const int ncols = (DELTA && mode == 1) ? dv + dk : dv;
   const int col = c0 + cl;
-  const bool col_ok = col < dv;
+  const bool col_ok = col < ncols;
   const int kh = hd / (H / p.G);  // the head's q/k head (delta rule) or B/C group (state space)
-  const long in_head = (static_cast<long>(hd) * dv + (col_ok ? col : 0)) * dk + rp * R;
+  const long in_head = (static_cast<long>(hd) * dv + (col < dv ? col : 0)) * dk + rp * R;
   const long sc_at = (static_cast<long>(s) * np + pc) * (static_cast<long>(H) * dv * dk);
   float* slot = p.state + static_cast<long>(p.state_rows[s]) * p.state_stride + p.off;
   const float* Sin = (mode == 2 ? p.sc_start + sc_at : slot) + in_head;
-  float* Sg = (mode == 1 ? p.sc_local + sc_at : slot) + in_head;
+  float* Sg = mode == 1 ? p.sc_local + (static_cast<long>(s) * np + pc) * (static_cast<long>(H) * ncols * dk) +
+                              (static_cast<long>(hd) * ncols + (col_ok ? col : 0)) * dk + rp * R
+                        : slot + in_head;
   const bool write_state = mode != 2 || te == qlen_all;
   const bool run_in = rp * R + R <= dk;
   float S[R];
@@ -177,7 +188,11 @@ __global__ void __launch_bounds__(256) column_scan_kernel(const ScanArgs p, int 
         if (rp * R + i < dk) S[i] = Sin[i];
     }
   }
-  float dsum = 0.f;  // mode 1: this thread's share of the piece's summed decay exponents
+  if (DELTA && mode == 1 && col >= dv) {
+#pragma unroll
+    for (int i = 0; i < R; ++i) S[i] = rp * R + i == col - dv ? 1.f : 0.f;
+  }
+  float dsum = 0.f;  // state space, mode 1: this thread's share of the piece's summed decay exponents
   const float eA = expf(p.A_log[hd]);
   const float Dh = DELTA ? 0.f : p.D[hd];
   float bias[DELTA ? R : 1];
@@ -281,7 +296,7 @@ __global__ void __launch_bounds__(256) column_scan_kernel(const ScanArgs p, int 
   __syncthreads();
   if (mode != 1 && cl < prev_nt && c0 + rp < dv)
     p.out[static_cast<long>(row0 + prev_t0 + cl) * HV + hd * dv + c0 + rp] = so[cl][rp];
-  if (mode == 1 && blockIdx.z == 0) {  // the piece's decay: exp(-sum) carries a state across it
+  if (!DELTA && mode == 1 && blockIdx.z == 0) {  // the piece's decay: exp(-sum) carries a state across it
     if (rp == 0) sa[cl] = dsum;
     __syncthreads();
     if (tid == 0) {
@@ -327,7 +342,8 @@ __global__ void __launch_bounds__(256) column_chain_kernel(const ScanArgs p) {
 
 template <typename T, bool DELTA>
 static bool launch_cs(const ScanArgs& a, int S, hipStream_t st) {
-  const dim3 grid(S * a.npieces, a.H, (a.dv + kCols - 1) / kCols), block(256);
+  const int ncols = (DELTA && a.mode == 1) ? a.dv + a.dk : a.dv;
+  const dim3 grid(S * a.npieces, a.H, (ncols + kCols - 1) / kCols), block(256);
   const int R = a.dk <= 32 ? 2 : a.dk <= 64 ? 4 : a.dk <= 128 ? 8 : 16;
   // which operands' runs of R elements are aligned to their size (16 bytes at most): 1 k, 2 q, 4 a, 8 state
   const size_t es = sizeof(T), al = std::min<size_t>(16, R * es), sal = std::min<size_t>(16, R * 4);
@@ -357,12 +373,15 @@ static bool launch_pass(const ScanArgs& a, int S, bool delta, bool bf, hipStream
 bool launch_column_scan(const ScanArgs& a0, int S, bool delta, bool bf, hipStream_t st) {
   if (S == 0 || a0.n_rows == 0) return true;
   ScanArgs a = a0;
-  if (delta || a.npieces <= 1) {  // the delta rule's step is no diagonal map: its chunks are walked whole
+  if (a.npieces <= 1) {
     a.mode = 0;
     a.piece = 1;
     a.npieces = 1;
     return launch_pass(a, S, delta, bf, st);
   }
+  // the delta rule's step is no diagonal map of the state: the caller runs its passes one by one and
+  // chains the pieces with matrix products in between (mxserve/ops/seqmix.py delta_scan)
+  if (delta) return (a.mode == 1 || a.mode == 2) && launch_pass(a, S, true, bf, st);
   a.mode = 1;
   if (!launch_pass(a, S, false, bf, st)) return false;
   const long per_head = static_cast<long>(a.dv) * a.dk;

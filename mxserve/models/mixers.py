@@ -399,7 +399,7 @@ class GatedDeltaRule(Mixer):
         g = ops.linear(g1.contiguous(), w[p + "g2"])
         o = seqmix.delta_scan(c[:, :n], c[:, n:2 * n], c[:, 2 * n:], b, a, w[p + "dt_bias"], w[p + "A_log"], ctx.state,
                               md.state_rows, soff, md.query_start_loc, md.seq_lens, self.heads, self.G, self.dk, self.dv,
-                              self.dk ** -0.5, self.unit_eps)
+                              self.dk ** -0.5, self.unit_eps, max_query_len=md.max_query_len)
         return seqmix.gated_norm(o, g, w[p + "norm"], ctx.eps, self.heads, "sigmoid", False, h.dtype, out_scale, out)
 
     def forward(self, parts: list, h: torch.Tensor, w: dict, ctx: StepContext, koff: int, voff: int, soff: int):

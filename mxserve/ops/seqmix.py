@@ -474,23 +474,48 @@ def ssd_scan(x: torch.Tensor, B: torch.Tensor, C: torch.Tensor, dt: torch.Tensor
     return out.reshape(T, H * P)
 
 
+DELTA_MIN_PIECES = 4  # a split delta-rule scan does three times the work: fewer pieces do not pay
+
+
 def delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, beta: torch.Tensor, a: torch.Tensor,
                dt_bias: torch.Tensor, A_log: torch.Tensor, state: torch.Tensor, state_rows: torch.Tensor, off: int,
                qsl: torch.Tensor, seq_lens: torch.Tensor, num_heads: int, qk_heads: int, dk: int, dv: int,
-               q_scale: float, unit_eps: float = 1e-6) -> torch.Tensor:
+               q_scale: float, unit_eps: float = 1e-6, max_query_len: int = 0) -> torch.Tensor:
     """Gated delta rule with one decay per head and key channel.  q, k [T, G*dk] are made unit vectors
     per head (x / sqrt(sum x^2 + unit_eps)), q also times q_scale; head h reads q/k head h // (H / G).
         g = exp(-exp(A_log_h) softplus(a + dt_bias))   [H, dk]      b = sigmoid(beta)   [H]
         S = diag(g) S;   u = b (v - S^T k);   S = S + k u^T;   o = S^T q
     so the read-out sees the token's own write.  v [T, H*dv], beta [T, H], a [T, H*dk] (row-strided
     views); dt_bias fp32 [H*dk], A_log fp32 [H].  Returns o fp32 [T, H*dv]; S (fp32, stored [H, dv, dk])
-    stays in the sequence's slot."""
+    stays in the sequence's slot.
+    max_query_len: the step's longest chunk (host int).  A token maps the state as S -> A_t S + b_t with
+    A_t = (I - b k k^T) diag(g), so a piece of tokens maps it as S -> P S + L: long chunks are cut into
+    pieces that run side by side, pass 1 giving every piece's L (end state from an empty start) and P
+    (dk more state columns started as the identity and fed no values), the states at the pieces'
+    starts following by one fp32 matrix product per piece, pass 2 writing the outputs.  Three times
+    the multiply-adds, but DELTA_MIN_PIECES or more pieces at once instead of one serial walk."""
     T = q.shape[0]
     H, G = num_heads, qk_heads
     if _gpu(q):
         out = torch.empty(T, H * dv, dtype=torch.float32, device=q.device)
-        ext().delta_scan(out, q, k, v, beta, a, dt_bias, A_log, state, state_rows, int(off), qsl, seq_lens, H, G, dk,
-                         dv, float(q_scale), float(unit_eps))
+        S = seq_lens.numel()
+        args = (out, q, k, v, beta, a, dt_bias, A_log, state, state_rows, int(off), qsl, seq_lens, H, G, dk, dv,
+                float(q_scale), float(unit_eps))
+        piece, npieces, _, _ = _scan_split(S, T, max_query_len, H * (dv + dk) * dk, H, 4 * (dv + dk), q.device)
+        if npieces < DELTA_MIN_PIECES:
+            ext().delta_scan(*args, 0, 1, 1, None, None)
+            return out
+        n = H * dv * dk
+        loc = torch.empty(S, npieces, H, dv + dk, dk, dtype=torch.float32, device=q.device)
+        start = torch.empty(S, npieces, H * dv, dk, dtype=torch.float32, device=q.device)
+        ext().delta_scan(*args, 1, piece, npieces, loc, start)
+        first = (seq_lens - (qsl[1:] - qsl[:-1]) <= 0).view(S, 1, 1)
+        slot = state.index_select(0, state_rows.long())[:, off:off + n].view(S, H * dv, dk)
+        start[:, 0] = torch.where(first, torch.zeros((), dtype=torch.float32, device=q.device), slot)
+        for p in range(npieces - 1):  # St' = St Pt + Lt in the transposed storage, batched over sequences and heads
+            start[:, p + 1] = torch.baddbmm(loc[:, p, :, :dv].reshape(S * H, dv, dk), start[:, p].reshape(S * H, dv, dk),
+                                            loc[:, p, :, dv:].reshape(S * H, dk, dk)).view(S, H * dv, dk)
+        ext().delta_scan(*args, 2, piece, npieces, loc, start)
         return out
     out = torch.zeros(T, H, dv, dtype=torch.float32)
     rep = H // G

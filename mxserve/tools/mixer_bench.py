@@ -244,7 +244,7 @@ def tapasun_rooflines(width: int, prompt: int, batch: int, context: int) -> list
                 aa = rnd(T, Hh * d1)
                 cb = torch.zeros(Hh * d1, device=dev)
                 fn = lambda: seqmix.delta_scan(qq, kk, vv, bb, aa, cb, hb, state, rows, 0, qsl, seq, Hh, Gg, d1, d2,  # noqa: E731
-                                               d1 ** -0.5)
+                                               d1 ** -0.5, max_query_len=T // S)
                 extra = T * Hh * d1
             t = _time(fn, 5)
             entry(f"{name}/{mode}", t, fl * T * Hh * d1 * d2, PEAK_F32,

@@ -166,6 +166,27 @@ def test_state_space_long_chunks(dev, portions):
 
 
 @pytest.mark.parametrize("dev", DEVS)
+@pytest.mark.parametrize("portions", [[300], [129, 171], [7, 290, 3], [150, 1, 149]])
+def test_delta_rule_long_chunks(dev, portions):
+    """The same for the delta rule, whose pieces are chained through their transition matrices."""
+    _skip(dev)
+    from mxserve.models.tapasun import build_mixer
+    width, T = 64, 300
+    h = torch.randn(T, width, generator=torch.Generator().manual_seed(6))
+    mc = parallel(rheads=4, rkv=2, rdim=24, rvdim=40, conv=3)["mixer"]
+    m = build_mixer("parallel", "m.", width, mc).right
+    g = torch.Generator().manual_seed(7)
+    shapes = {name: (rows, width) for name, rows in m.proj_rows()}
+    shapes.update(m.extra_shapes())
+    w = {k: torch.randn(s, generator=g) * (s[-1] ** -0.5 if len(s) > 1 else 1.0) for k, s in shapes.items()}
+    w["m.right.A_log"] = w["m.right.A_log"] - 3.0  # slow decays: what a piece inherits matters to its end
+    w["m.right.dt_bias"] = w["m.right.dt_bias"] - 1.0
+    wn = {k: v.double().numpy() for k, v in w.items()}
+    want = _oracle_steps(to.GatedDeltaRule(mc["right"], wn, "m.right.", EPS), h.double().numpy())
+    _check(_run_mixers([m], [w], h, dev, portions)[0], want, 1e-4)
+
+
+@pytest.mark.parametrize("dev", DEVS)
 @pytest.mark.parametrize("portions", PORTIONS)
 def test_rotary_attention_mixer_and_shared_pages(dev, portions):
     """An attention layer with keys of its own and a second one that reads the first one's pages with
