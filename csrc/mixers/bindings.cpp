@@ -338,7 +338,7 @@ void column_scan(bool delta, at::Tensor out, at::Tensor q, at::Tensor k, at::Ten
                  at::Tensor dt_bias, at::Tensor A_log, OptT D, at::Tensor state, at::Tensor state_rows, int64_t off,
                  at::Tensor qsl, at::Tensor seq_lens, int64_t H, int64_t G, int64_t dk, int64_t dv, double q_scale,
                  double unit_eps, int64_t piece = 1, int64_t npieces = 1, OptT sc_local = OptT(), OptT sc_start = OptT(),
-                 OptT sc_decay = OptT(), int64_t mode = 0) {
+                 OptT sc_decay = OptT(), int64_t mode = 0, int64_t max_q = 0) {
   const bool bf = is_bf(q);
   const int64_t T = q.size(0), S = seq_lens.numel();
   TORCH_CHECK(G >= 1 && H % G == 0, "heads must divide over the q/k heads (groups)");
@@ -379,6 +379,7 @@ void column_scan(bool delta, at::Tensor out, at::Tensor q, at::Tensor k, at::Ten
   p.unit_eps = static_cast<float>(unit_eps);
   p.piece = 1;
   p.npieces = 1;
+  p.max_q = (max_q == 1 && T == S) ? 1 : 0;  // every sequence brings one row
   if (npieces > 1) {  // pieces side by side: scratch [S, npieces, state] twice and [S, npieces, H]
     TORCH_CHECK(piece >= 16 && sc_local.has_value() && sc_start.has_value() && (delta || sc_decay.has_value()),
                 "a split scan needs its scratch pools");
@@ -399,17 +400,17 @@ void column_scan(bool delta, at::Tensor out, at::Tensor q, at::Tensor k, at::Ten
 void ssd_scan(at::Tensor out, at::Tensor x, at::Tensor B, at::Tensor C, at::Tensor dt, at::Tensor dt_bias, at::Tensor A_log,
               at::Tensor D, at::Tensor state, at::Tensor state_rows, int64_t off, at::Tensor qsl, at::Tensor seq_lens,
               int64_t H, int64_t G, int64_t N, int64_t P, int64_t piece, int64_t npieces, OptT sc_local, OptT sc_start,
-              OptT sc_decay) {
+              OptT sc_decay, int64_t max_q) {
   column_scan(false, out, C, B, x, dt, OptT(), dt_bias, A_log, OptT(D), state, state_rows, off, qsl, seq_lens, H, G, N, P,
-              1.0, 0.0, piece, npieces, sc_local, sc_start, sc_decay);
+              1.0, 0.0, piece, npieces, sc_local, sc_start, sc_decay, 0, max_q);
 }
 
 void delta_scan(at::Tensor out, at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor beta, at::Tensor a, at::Tensor dt_bias,
                 at::Tensor A_log, at::Tensor state, at::Tensor state_rows, int64_t off, at::Tensor qsl, at::Tensor seq_lens,
                 int64_t H, int64_t G, int64_t dk, int64_t dv, double q_scale, double unit_eps, int64_t mode, int64_t piece,
-                int64_t npieces, OptT sc_local, OptT sc_start) {
+                int64_t npieces, OptT sc_local, OptT sc_start, int64_t max_q) {
   column_scan(true, out, q, k, v, beta, OptT(a), dt_bias, A_log, OptT(), state, state_rows, off, qsl, seq_lens, H, G, dk, dv,
-              q_scale, unit_eps, piece, npieces, sc_local, sc_start, OptT(), mode);
+              q_scale, unit_eps, piece, npieces, sc_local, sc_start, OptT(), mode, max_q);
 }
 
 }  // namespace

@@ -25,6 +25,7 @@ struct ScanArgs {
   const int* qsl;
   const int* seq_lens;
   int n_rows, H, G, dk, dv;
+  int max_q;  // the step's longest chunk; 1: single tokens only (a smaller stage)
   float q_scale, unit_eps;
   // state space, long chunks cut into pieces that run side by side: mode 0 whole chunk, state from and
   // to the slot; mode 1 a piece from an empty state, its end state to sc_local and its summed decay

@@ -96,12 +96,12 @@ template <int R> __device__ __forceinline__ void store_run(float* p, const float
 // token tid / 16; the run is the one whose rows it owns in the recurrence), one value element and the
 // token's scalar.  The loads of a stage are issued before the 16 tokens of the stage before it are
 // walked, so their latency hides behind that walk.
-template <int R, bool DELTA> struct StageRegs {
-  float k[R], q[R], a[DELTA ? R : 1], v, b;
+template <int R, bool DELTA, int CG> struct StageRegs {
+  float k[R], q[R], a[DELTA ? R : 1], v[CG], b;
 };
 
-template <typename T, int R, bool DELTA>
-__device__ __forceinline__ void load_stage(StageRegs<R, DELTA>& r, const ScanArgs& p, long row, bool ok, int kh, int hd,
+template <typename T, int R, bool DELTA, int CG>
+__device__ __forceinline__ void load_stage(StageRegs<R, DELTA, CG>& r, const ScanArgs& p, long row, bool ok, int kh, int hd,
                                            int rp, int vcol, int flags) {
   const T* qp = static_cast<const T*>(p.q);
   const T* kp = static_cast<const T*>(p.k);
@@ -115,7 +115,8 @@ __device__ __forceinline__ void load_stage(StageRegs<R, DELTA>& r, const ScanArg
     r.q[i] = 0.f;
     if (DELTA) r.a[i] = 0.f;
   }
-  r.v = 0.f;
+#pragma unroll
+  for (int j = 0; j < CG; ++j) r.v[j] = 0.f;
   r.b = 0.f;
   if (!ok) return;
   if (d0 + R <= p.dk) {
@@ -132,21 +133,28 @@ __device__ __forceinline__ void load_stage(StageRegs<R, DELTA>& r, const ScanArg
       }
     }
   }
-  if (vcol < p.dv) r.v = ldf(vp + row * p.v_stride + hd * p.dv + vcol);
+#pragma unroll
+  for (int j = 0; j < CG; ++j)
+    if (vcol + j * kCols < p.dv) r.v[j] = ldf(vp + row * p.v_stride + hd * p.dv + vcol + j * kCols);
   r.b = ldf(bp + row * p.beta_stride + hd);
 }
 
-template <typename T, int R, bool DELTA>
+// ST: tokens per stage, 16, or 1 for steps of single tokens only.  CG: groups of 16 columns a workgroup
+// takes, each thread one column of every group: a step of single tokens is a read and a write of the
+// state and little else, so its workgroups take 64 columns and have four times the bytes in flight.
+template <typename T, int R, bool DELTA, int ST, int CG>
 __global__ void __launch_bounds__(256) column_scan_kernel(const ScanArgs p, int flags) {
   constexpr int DK = 16 * R;  // padded key size
-  __shared__ __attribute__((aligned(16))) float sk[kST][DK];
-  __shared__ __attribute__((aligned(16))) float sq[kST][DK];
-  __shared__ __attribute__((aligned(16))) float sg[DELTA ? kST : 1][DELTA ? DK : 4];
-  __shared__ float sv[kST][kCols];
-  __shared__ float so[kST][kCols];
-  __shared__ float sb[kST], sa[kST];
+  __shared__ __attribute__((aligned(16))) float sk[ST][DK];
+  __shared__ __attribute__((aligned(16))) float sq[ST][DK];
+  __shared__ __attribute__((aligned(16))) float sg[DELTA ? ST : 1][DELTA ? DK : 4];
+  constexpr int WC = kCols * CG;  // columns per workgroup
+  __shared__ float sv[ST][WC];
+  __shared__ float so[ST][WC];
+  __shared__ float sb[ST], sa[kST];
   const int mode = p.mode, np = p.npieces;
-  const int s = blockIdx.x / np, pc = blockIdx.x - s * np, hd = blockIdx.y, c0 = blockIdx.z * kCols;
+  // neighbouring workgroups take neighbouring columns of one head's state: consecutive memory
+  const int s = blockIdx.z / np, pc = blockIdx.z - s * np, hd = blockIdx.y, c0 = blockIdx.x * WC;
   const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
   // recurrence: the thread owns rows rp*R.. of column cl.  staging: run rp of token cl.
   const int rp = lane & 15, cl = wid * 4 + (lane >> 4);
@@ -164,33 +172,34 @@ __global__ void __launch_bounds__(256) column_scan_kernel(const ScanArgs p, int 
   // transition matrix (the state at the piece's end is that matrix times the state at its start, plus
   // the end state from an empty start)
   const int ncols = (DELTA && mode == 1) ? dv + dk : dv;
-  const int col = c0 + cl;
-  const bool col_ok = col < ncols;
   const int kh = hd / (H / p.G);  // the head's q/k head (delta rule) or B/C group (state space)
-  const long in_head = (static_cast<long>(hd) * dv + (col < dv ? col : 0)) * dk + rp * R;
   const long sc_at = (static_cast<long>(s) * np + pc) * (static_cast<long>(H) * dv * dk);
   float* slot = p.state + static_cast<long>(p.state_rows[s]) * p.state_stride + p.off;
-  const float* Sin = (mode == 2 ? p.sc_start + sc_at : slot) + in_head;
-  float* Sg = mode == 1 ? p.sc_local + (static_cast<long>(s) * np + pc) * (static_cast<long>(H) * ncols * dk) +
-                              (static_cast<long>(hd) * ncols + (col_ok ? col : 0)) * dk + rp * R
-                        : slot + in_head;
+  const float* Sin0 = mode == 2 ? p.sc_start + sc_at : slot;
+  float* Sout0 = mode == 1 ? p.sc_local + (static_cast<long>(s) * np + pc) * (static_cast<long>(H) * ncols * dk) : slot;
+  const int out_cols = mode == 1 ? ncols : dv;  // columns per head where the state goes
   const bool write_state = mode != 2 || te == qlen_all;
   const bool run_in = rp * R + R <= dk;
-  float S[R];
+  float S[CG][R];
 #pragma unroll
-  for (int i = 0; i < R; ++i) S[i] = 0.f;
-  if (!fresh && col_ok) {
-    if (run_in) {
-      load_run<R>(Sin, S, flags & 8);
-    } else {
+  for (int j = 0; j < CG; ++j) {  // every group's loads are issued before any is waited for
+    const int col = c0 + j * kCols + cl;
 #pragma unroll
-      for (int i = 0; i < R; ++i)
-        if (rp * R + i < dk) S[i] = Sin[i];
+    for (int i = 0; i < R; ++i) S[j][i] = 0.f;
+    if (!fresh && col < dv) {
+      const float* Sin = Sin0 + (static_cast<long>(hd) * dv + col) * dk + rp * R;
+      if (run_in) {
+        load_run<R>(Sin, S[j], flags & 8);
+      } else {
+#pragma unroll
+        for (int i = 0; i < R; ++i)
+          if (rp * R + i < dk) S[j][i] = Sin[i];
+      }
     }
-  }
-  if (DELTA && mode == 1 && col >= dv) {
+    if (DELTA && mode == 1 && col >= dv) {
 #pragma unroll
-    for (int i = 0; i < R; ++i) S[i] = rp * R + i == col - dv ? 1.f : 0.f;
+      for (int i = 0; i < R; ++i) S[j][i] = rp * R + i == col - dv ? 1.f : 0.f;
+    }
   }
   float dsum = 0.f;  // state space, mode 1: this thread's share of the piece's summed decay exponents
   const float eA = expf(p.A_log[hd]);
@@ -203,16 +212,22 @@ __global__ void __launch_bounds__(256) column_scan_kernel(const ScanArgs p, int 
     bias[0] = p.dt_bias[hd];
   }
   const int HV = H * dv;
-  StageRegs<R, DELTA> rg;
-  load_stage<T, R, DELTA>(rg, p, row0 + cl, cl < qlen, kh, hd, rp, c0 + rp, flags);
+  StageRegs<R, DELTA, CG> rg;
+  load_stage<T, R, DELTA, CG>(rg, p, row0 + cl, cl < ST && cl < qlen, kh, hd, rp, c0 + rp, flags);
   int prev_t0 = -1, prev_nt = 0;
-  for (int t0 = 0; t0 < qlen; t0 += kST) {
-    const int nt = min(kST, qlen - t0);
+  for (int t0 = 0; t0 < qlen; t0 += ST) {
+    const int nt = min(ST, qlen - t0);
     __syncthreads();  // the previous stage's reads of the staged vectors and writes of so are done
-    if (mode != 1 && prev_t0 >= 0 && cl < prev_nt && c0 + rp < dv)
-      p.out[static_cast<long>(row0 + prev_t0 + cl) * HV + hd * dv + c0 + rp] = so[cl][rp];
+    if (mode != 1 && prev_t0 >= 0 && cl < prev_nt) {
+#pragma unroll
+      for (int j = 0; j < CG; ++j)
+        if (c0 + j * kCols + rp < dv)
+          p.out[static_cast<long>(row0 + prev_t0 + cl) * HV + hd * dv + c0 + j * kCols + rp] = so[cl][j * kCols + rp];
+    }
     // this stage's registers -> LDS, with everything that is per token and head applied
-    if (DELTA) {
+    if (cl >= ST) {
+      // ST = 1: the other fifteen token rows of the staging layout have nothing to bring
+    } else if (DELTA) {
       float ssk = 0.f, ssq = 0.f;
 #pragma unroll
       for (int i = 0; i < R; ++i) {
@@ -240,34 +255,40 @@ __global__ void __launch_bounds__(256) column_scan_kernel(const ScanArgs p, int 
         if (cl < nt) dsum += eA * dt;
       }
     }
-    sv[cl][rp] = rg.v;
+    if (cl < ST) {
+#pragma unroll
+      for (int j = 0; j < CG; ++j) sv[cl][j * kCols + rp] = rg.v[j];
+    }
     __syncthreads();
-    if (t0 + kST < qlen)  // the next stage's loads fly while this stage's tokens are walked
-      load_stage<T, R, DELTA>(rg, p, row0 + t0 + kST + cl, t0 + kST + cl < qlen, kh, hd, rp, c0 + rp, flags);
+    if (t0 + ST < qlen)  // the next stage's loads fly while this stage's tokens are walked
+      load_stage<T, R, DELTA, CG>(rg, p, row0 + t0 + ST + cl, cl < ST && t0 + ST + cl < qlen, kh, hd, rp, c0 + rp, flags);
     auto token = [&](int tt) {
-      const float vj = sv[tt][cl];
       const float* kr = &sk[tt][rp * R];
       const float* qr = &sq[tt][rp * R];
+#pragma unroll
+      for (int j = 0; j < CG; ++j) {
+      float* Sj = S[j];
+      const float vj = sv[tt][j * kCols + cl];
       float o;
       if (DELTA) {
         const float* gr = &sg[tt][rp * R];
         float p0 = 0.f, p1 = 0.f;
 #pragma unroll
         for (int i = 0; i < R; i += 2) {
-          S[i] *= gr[i];
-          S[i + 1] *= gr[i + 1];
-          p0 += S[i] * kr[i];
-          p1 += S[i + 1] * kr[i + 1];
+          Sj[i] *= gr[i];
+          Sj[i + 1] *= gr[i + 1];
+          p0 += Sj[i] * kr[i];
+          p1 += Sj[i + 1] * kr[i + 1];
         }
         const float u = sb[tt] * (vj - row16_sum(p0 + p1));
         p0 = 0.f;
         p1 = 0.f;
 #pragma unroll
         for (int i = 0; i < R; i += 2) {
-          S[i] += kr[i] * u;
-          S[i + 1] += kr[i + 1] * u;
-          p0 += S[i] * qr[i];
-          p1 += S[i + 1] * qr[i + 1];
+          Sj[i] += kr[i] * u;
+          Sj[i + 1] += kr[i + 1] * u;
+          p0 += Sj[i] * qr[i];
+          p1 += Sj[i + 1] * qr[i + 1];
         }
         o = row16_sum(p0 + p1);
       } else {
@@ -275,18 +296,19 @@ __global__ void __launch_bounds__(256) column_scan_kernel(const ScanArgs p, int 
         float p0 = 0.f, p1 = 0.f;
 #pragma unroll
         for (int i = 0; i < R; i += 2) {
-          S[i] = a * S[i] + xb * kr[i];
-          S[i + 1] = a * S[i + 1] + xb * kr[i + 1];
-          p0 += S[i] * qr[i];
-          p1 += S[i + 1] * qr[i + 1];
+          Sj[i] = a * Sj[i] + xb * kr[i];
+          Sj[i + 1] = a * Sj[i + 1] + xb * kr[i + 1];
+          p0 += Sj[i] * qr[i];
+          p1 += Sj[i + 1] * qr[i + 1];
         }
         o = row16_sum(p0 + p1) + Dh * vj;
       }
-      if (rp == 0) so[tt][cl] = o;
+      if (rp == 0) so[tt][j * kCols + cl] = o;
+      }
     };
-    if (nt == kST) {
+    if (ST > 1 && nt == ST) {
 #pragma unroll 4
-      for (int tt = 0; tt < kST; ++tt) token(tt);
+      for (int tt = 0; tt < ST; ++tt) token(tt);
     } else {
       for (int tt = 0; tt < nt; ++tt) token(tt);
     }
@@ -294,9 +316,13 @@ __global__ void __launch_bounds__(256) column_scan_kernel(const ScanArgs p, int 
     prev_nt = nt;
   }
   __syncthreads();
-  if (mode != 1 && cl < prev_nt && c0 + rp < dv)
-    p.out[static_cast<long>(row0 + prev_t0 + cl) * HV + hd * dv + c0 + rp] = so[cl][rp];
-  if (!DELTA && mode == 1 && blockIdx.z == 0) {  // the piece's decay: exp(-sum) carries a state across it
+  if (mode != 1 && cl < prev_nt) {
+#pragma unroll
+    for (int j = 0; j < CG; ++j)
+      if (c0 + j * kCols + rp < dv)
+        p.out[static_cast<long>(row0 + prev_t0 + cl) * HV + hd * dv + c0 + j * kCols + rp] = so[cl][j * kCols + rp];
+  }
+  if (!DELTA && mode == 1 && blockIdx.x == 0) {  // the piece's decay: exp(-sum) carries a state across it
     if (rp == 0) sa[cl] = dsum;
     __syncthreads();
     if (tid == 0) {
@@ -305,13 +331,19 @@ __global__ void __launch_bounds__(256) column_scan_kernel(const ScanArgs p, int 
       p.sc_decay[(static_cast<long>(s) * np + pc) * H + hd] = t;
     }
   }
-  if (col_ok && write_state) {
-    if (run_in) {
-      store_run<R>(Sg, S, flags & 8);
-    } else {
+  if (write_state) {
 #pragma unroll
-      for (int i = 0; i < R; ++i)
-        if (rp * R + i < dk) Sg[i] = S[i];
+    for (int j = 0; j < CG; ++j) {
+      const int col = c0 + j * kCols + cl;
+      if (col >= out_cols) continue;
+      float* Sg = Sout0 + (static_cast<long>(hd) * out_cols + col) * dk + rp * R;
+      if (run_in) {
+        store_run<R>(Sg, S[j], flags & 8);
+      } else {
+#pragma unroll
+        for (int i = 0; i < R; ++i)
+          if (rp * R + i < dk) Sg[i] = S[j][i];
+      }
     }
   }
 }
@@ -343,7 +375,9 @@ __global__ void __launch_bounds__(256) column_chain_kernel(const ScanArgs p) {
 template <typename T, bool DELTA>
 static bool launch_cs(const ScanArgs& a, int S, hipStream_t st) {
   const int ncols = (DELTA && a.mode == 1) ? a.dv + a.dk : a.dv;
-  const dim3 grid(S * a.npieces, a.H, (ncols + kCols - 1) / kCols), block(256);
+  const int wc = a.max_q == 1 ? 4 * kCols : kCols;  // columns per workgroup
+  const dim3 grid((ncols + wc - 1) / wc, a.H, S * a.npieces), block(256);
+  if (grid.z > 65535u) return false;
   const int R = a.dk <= 32 ? 2 : a.dk <= 64 ? 4 : a.dk <= 128 ? 8 : 16;
   // which operands' runs of R elements are aligned to their size (16 bytes at most): 1 k, 2 q, 4 a, 8 state
   const size_t es = sizeof(T), al = std::min<size_t>(16, R * es), sal = std::min<size_t>(16, R * 4);
@@ -354,7 +388,11 @@ static bool launch_cs(const ScanArgs& a, int S, hipStream_t st) {
   if (reinterpret_cast<uintptr_t>(a.state) % sal == 0 && (a.state_stride * 4) % sal == 0 && (a.off * 4) % sal == 0 &&
       (a.dk * 4) % sal == 0)
     flags |= 8;
-#define MIX_CS(R) hipLaunchKernelGGL((column_scan_kernel<T, R, DELTA>), grid, block, 0, st, a, flags)
+#define MIX_CS(R)                                                                                              \
+  do {                                                                                                         \
+    if (a.max_q == 1) hipLaunchKernelGGL((column_scan_kernel<T, R, DELTA, 1, 4>), grid, block, 0, st, a, flags);  \
+    else hipLaunchKernelGGL((column_scan_kernel<T, R, DELTA, kST, 1>), grid, block, 0, st, a, flags);             \
+  } while (0)
   if (a.dk <= 32) MIX_CS(2);
   else if (a.dk <= 64) MIX_CS(4);
   else if (a.dk <= 128) MIX_CS(8);

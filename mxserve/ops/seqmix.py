@@ -451,7 +451,7 @@ def ssd_scan(x: torch.Tensor, B: torch.Tensor, C: torch.Tensor, dt: torch.Tensor
         piece, npieces, loc, start = _scan_split(seq_lens.numel(), T, max_query_len, H * N * P, H, 4 * P, x.device)
         dec = torch.empty(seq_lens.numel() * npieces * H, dtype=torch.float32, device=x.device) if npieces > 1 else None
         ext().ssd_scan(out, x, B, C, dt, dt_bias, A_log, D, state, state_rows, int(off), qsl, seq_lens, H, groups, N, P,
-                       piece, npieces, loc, start, dec)
+                       piece, npieces, loc, start, dec, int(max_query_len))
         return out
     out = torch.zeros(T, H, P, dtype=torch.float32)
     xf = x.float().reshape(T, H, P)
@@ -503,19 +503,19 @@ def delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, beta: torch.Te
                 float(q_scale), float(unit_eps))
         piece, npieces, _, _ = _scan_split(S, T, max_query_len, H * (dv + dk) * dk, H, 4 * (dv + dk), q.device)
         if npieces < DELTA_MIN_PIECES:
-            ext().delta_scan(*args, 0, 1, 1, None, None)
+            ext().delta_scan(*args, 0, 1, 1, None, None, int(max_query_len))
             return out
         n = H * dv * dk
         loc = torch.empty(S, npieces, H, dv + dk, dk, dtype=torch.float32, device=q.device)
         start = torch.empty(S, npieces, H * dv, dk, dtype=torch.float32, device=q.device)
-        ext().delta_scan(*args, 1, piece, npieces, loc, start)
+        ext().delta_scan(*args, 1, piece, npieces, loc, start, int(max_query_len))
         first = (seq_lens - (qsl[1:] - qsl[:-1]) <= 0).view(S, 1, 1)
         slot = state.index_select(0, state_rows.long())[:, off:off + n].view(S, H * dv, dk)
         start[:, 0] = torch.where(first, torch.zeros((), dtype=torch.float32, device=q.device), slot)
         for p in range(npieces - 1):  # St' = St Pt + Lt in the transposed storage, batched over sequences and heads
             start[:, p + 1] = torch.baddbmm(loc[:, p, :, :dv].reshape(S * H, dv, dk), start[:, p].reshape(S * H, dv, dk),
                                             loc[:, p, :, dv:].reshape(S * H, dk, dk)).view(S, H * dv, dk)
-        ext().delta_scan(*args, 2, piece, npieces, loc, start)
+        ext().delta_scan(*args, 2, piece, npieces, loc, start, int(max_query_len))
         return out
     out = torch.zeros(T, H, dv, dtype=torch.float32)
     rep = H // G
