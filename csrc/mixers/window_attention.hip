@@ -294,7 +294,8 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(
   const int qt0 = blockIdx.x * 64 + wid * 16;  // this wave's first query row inside the chunk
   if (qt0 >= qlen) return;                     // wave-uniform (no workgroup barrier is used below)
   const int nq = min(16, qlen - qt0);
-  const int pos0 = min(max(seq_lens[s] - qlen + qt0, 0), bt_stride * 16 - 16);
+  // the tile's first position; its last row stays inside the block table whatever the metadata says
+  const int pos0 = min(max(seq_lens[s] - qlen + qt0, 0), bt_stride * 16 - nq);
   const int g = hd / (H / G);
   const int c = lane & 15, kg = lane >> 4;  // the lane's query (column) and its group of 4 keys / dims
   const int KS = dk >> 4, VT = dv >> 4;
