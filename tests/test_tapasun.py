@@ -415,6 +415,28 @@ def test_mixed_batches_reuse_pages_and_slots(base, dev, dtype, tol, eager):
     assert eng.kv.num_free() == eng.kv.num_blocks and not eng.runner._row_of
 
 
+@pytest.mark.parametrize("dev,dtype,tol", DEV_DTYPE_TOL)
+def test_request_that_fills_the_pool(tmp_path, dev, dtype, tol):
+    """A request three tokens short of the pool and of the longest sequence the engine admits, with head
+    sizes that take the matrix-core attention in bf16: its last portions end in partial tiles on the
+    last page of the block table."""
+    _skip(dev)
+    cfg = config([attention(heads=4, kv_heads=2, dim=64, vdim=64, dims=32, scale=0.125, mlp=128),
+                  parallel(heads=4, kv_heads=1, dim=32, vdim=32, dims=16, scale=0.18, rheads=2, rkv=2, rdim=32, rvdim=32,
+                           conv=4, mlp=None),
+                  attention(heads=4, kv_heads=2, dim=64, vdim=64, dims=32, scale=0.125, kv_from=0, mlp=128)],
+                 width=128, vocab=200)
+    w = write_checkpoint(tmp_path, cfg, seed=8)
+    t = _tokens(125, cfg["vocab"], 9)
+    want = _oracle_model(cfg, w, t)
+    eng = engine(tmp_path, dev, dtype, max_tokens=128)
+    for sizes in ([1000], [90, 35], [100, 19, 1], [64, 40, 21]):
+        steps = [[("a", p, False)] for p in cut(t, sizes)]
+        steps[-1] = [("a", steps[-1][0][1], True)]
+        _check(replay(eng, steps)["a"], want, tol)
+    assert eng.kv.num_free() == eng.kv.num_blocks
+
+
 VARIANTS = {
     "every_head_its_own_kv_and_group": config([attention(heads=3, kv_heads=3, dim=16, vdim=16, dims=16, scaling=None, mlp=64),
                                                mamba2(heads=2, vdim=16, state=16, groups=2, conv=2, norm_groups=2, mlp=None),
