@@ -383,6 +383,13 @@ class GatedDeltaRule(Mixer):
         p = self.p
         # one filter over q, k, v's channels, tap-major for the kernel
         w[p + "_conv"] = torch.cat([w.pop(p + "q.conv"), w.pop(p + "k.conv"), w.pop(p + "v.conv")]).t().contiguous()
+        # the second halves of the two low-rank pairs as one projection of [a1 h | g1 h]: a2 and g2 on the
+        # diagonal, zeros beside them (their products add exactly nothing)
+        a2, g2 = w.pop(p + "a2"), w.pop(p + "g2")
+        both = torch.zeros(a2.shape[0] + g2.shape[0], a2.shape[1] + g2.shape[1], dtype=a2.dtype, device=a2.device)
+        both[:a2.shape[0], :a2.shape[1]] = a2
+        both[a2.shape[0]:, a2.shape[1]:] = g2
+        w[p + "_ag2"] = both
         _fp32(w, p + "dt_bias")
         _fp32(w, p + "A_log")
 
@@ -395,8 +402,11 @@ class GatedDeltaRule(Mixer):
         qkv = torch.as_strided(q, (q.shape[0], self.conv_ch), q.stride(), q.storage_offset())
         c = seqmix.causal_conv(qkv, w[p + "_conv"], None, ctx.state, md.state_rows, soff + self.scan_floats,
                                md.query_start_loc, md.seq_lens, silu=True)
-        a = ops.linear(a1.contiguous(), w[p + "a2"])
-        g = ops.linear(g1.contiguous(), w[p + "g2"])
+        # a1 and g1 are neighbours too: one projection gives the decay pre-activations and the gate's
+        ra = a1.shape[1]
+        ag = ops.linear(torch.as_strided(a1, (a1.shape[0], ra + g1.shape[1]), a1.stride(), a1.storage_offset()).contiguous(),
+                        w[p + "_ag2"])
+        a, g = ag[:, :self.heads * self.dk], ag[:, self.heads * self.dk:]
         o = seqmix.delta_scan(c[:, :n], c[:, n:2 * n], c[:, 2 * n:], b, a, w[p + "dt_bias"], w[p + "A_log"], ctx.state,
                               md.state_rows, soff, md.query_start_loc, md.seq_lens, self.heads, self.G, self.dk, self.dv,
                               self.dk ** -0.5, self.unit_eps, max_query_len=md.max_query_len)
