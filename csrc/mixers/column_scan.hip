@@ -262,6 +262,7 @@ __global__ void __launch_bounds__(256) column_scan_kernel(const ScanArgs p, int 
     __syncthreads();
     if (t0 + ST < qlen)  // the next stage's loads fly while this stage's tokens are walked
       load_stage<T, R, DELTA, CG>(rg, p, row0 + t0 + ST + cl, cl < ST && t0 + ST + cl < qlen, kh, hd, rp, c0 + rp, flags);
+    const bool readout = mode != 1;  // pass 1 wants a piece's end state only
     auto token = [&](int tt) {
       const float* kr = &sk[tt][rp * R];
       const float* qr = &sq[tt][rp * R];
@@ -281,17 +282,23 @@ __global__ void __launch_bounds__(256) column_scan_kernel(const ScanArgs p, int 
           p1 += Sj[i + 1] * kr[i + 1];
         }
         const float u = sb[tt] * (vj - row16_sum(p0 + p1));
-        p0 = 0.f;
-        p1 = 0.f;
+        if (readout) {
+          p0 = 0.f;
+          p1 = 0.f;
 #pragma unroll
-        for (int i = 0; i < R; i += 2) {
-          Sj[i] += kr[i] * u;
-          Sj[i + 1] += kr[i + 1] * u;
-          p0 += Sj[i] * qr[i];
-          p1 += Sj[i + 1] * qr[i + 1];
+          for (int i = 0; i < R; i += 2) {
+            Sj[i] += kr[i] * u;
+            Sj[i + 1] += kr[i + 1] * u;
+            p0 += Sj[i] * qr[i];
+            p1 += Sj[i + 1] * qr[i + 1];
+          }
+          o = row16_sum(p0 + p1);
+        } else {
+#pragma unroll
+          for (int i = 0; i < R; ++i) Sj[i] += kr[i] * u;
+          o = 0.f;
         }
-        o = row16_sum(p0 + p1);
-      } else {
+      } else if (readout) {
         const float a = sa[tt], xb = sb[tt] * vj;
         float p0 = 0.f, p1 = 0.f;
 #pragma unroll
@@ -302,8 +309,13 @@ __global__ void __launch_bounds__(256) column_scan_kernel(const ScanArgs p, int 
           p1 += Sj[i + 1] * qr[i + 1];
         }
         o = row16_sum(p0 + p1) + Dh * vj;
+      } else {
+        const float a = sa[tt], xb = sb[tt] * vj;
+#pragma unroll
+        for (int i = 0; i < R; ++i) Sj[i] = a * Sj[i] + xb * kr[i];
+        o = 0.f;
       }
-      if (rp == 0) so[tt][j * kCols + cl] = o;
+      if (readout && rp == 0) so[tt][j * kCols + cl] = o;
       }
     };
     if (ST > 1 && nt == ST) {
